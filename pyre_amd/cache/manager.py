@@ -11,7 +11,8 @@ several). A *cell* is (entry, index in that list). Cells with the same needs for
   Which tensors a page holds, and how a page of each is laid out, is what the
   description says (the mixer's choice); the manager allocates
   ``[layers, pages, *page_shape]`` for each and knows nothing of their meaning.
-  A group with a window gives a page back as soon as no later query can see it.
+  A group with a window gives a page back as soon as no later query can see it (the pages of
+  the first tokens that such a window keeps visible stay).
   All groups share one page size, the engine's; a description that names another
   (``PagedCacheSpec.page_size``: a mixer whose kernels need pages of a particular size) is
   refused when the manager is made.
@@ -285,8 +286,9 @@ class CacheManager:
             # The next query sits at position req.length and sees keys > length - w.
             dead_upto = req.length - w  # keys <= dead_upto are never read again
             last_dead_page = (dead_upto + 1) // self.page_size - 1
+            kept_pages = -(-g.spec.keep_first // self.page_size)  # they hold the first tokens, which stay visible
             dead = []
-            for i in range(min(last_dead_page + 1, len(table))):
+            for i in range(kept_pages, min(last_dead_page + 1, len(table))):
                 if table[i] != RELEASED:
                     g.allocator.free(table[i])
                     dead.append(table[i])

@@ -1,0 +1,393 @@
+// Softmax attention without rotation whose positions enter through the scores: unit-norm
+// queries and keys, a cap on the scores, a learned bias by distance, a window that also keeps
+// the first tokens of the sequence, key and value heads of different sizes, and one gate per
+// head on the output. Three kernels over the paged cache k [pages, nkv, page, dk] and
+// v [pages, nkv, page, dv] (both one record per token), float32 or bfloat16 storage, all
+// arithmetic float32:
+//
+//   s(i, j) = (q_i . k_j) * scale;   s <- cap * tanh(s / cap)  (cap > 0);   s <- s + bias[head][min(i - j, far)]
+//   i sees j  iff  j <= i and (window == 0 or i - j < window or j < keep_first)
+//   out_i = gate_i * out_scale * sum_j softmax_j(s(i, .)) v_j
+//
+// `bias` is the table by distance that the host made of the model's buckets: [nq][far + 1] float32,
+// or null. `gate` is float32 [n][nq] (already squashed), or null.
+//
+// unit_qkv_write  finishes the input product of a step (partial sums), divides every query and key
+//                 head by its root mean square, stores queries, keys and values and the squashed gates.
+// attn_biased_tile    prompt portions: tiles of up to 32 consecutive tokens of a request, four query
+//                 heads of a key/value head per block, chunks of 32 keys through LDS, both products on
+//                 the matrix cores' float32 instruction (scores and weights stay float32).
+// attn_biased_single  single tokens: a block per (token, query head), the keys in spans of 128.
+//
+// Chunks start at multiples of 32 keys and spans at the token's first visible key, so the order of
+// every sum of a token depends on its own bounds alone.
+#include "pyre_api.h"
+#include "pyre_common.h"
+
+using namespace pyre;
+
+namespace {
+
+constexpr int kThreads = 256;
+
+// ---------------------------------------------------------------------------------------------
+template <typename TC>
+__global__ __launch_bounds__(kThreads) void unit_qkv_write_kernel(
+    const void* __restrict__ proj, int proj_dt, int n_partials, size_t partial_stride, int ld, int col0,
+    void* __restrict__ q_out, int q_dt, TC* __restrict__ k_cache, TC* __restrict__ v_cache,
+    float* __restrict__ gate_out, const int* __restrict__ slots, int nq, int nkv, int dk, int dv, int page_size,
+    int unit_norm, float eps, int gated, int write_kv) {
+  const int n = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const size_t in_row = static_cast<size_t>(n) * ld + col0;
+  const int slot = write_kv ? slots[n] : -1;
+  const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+
+  auto value = [&](int col) {
+    float v = 0.f;
+    for (int p = 0; p < n_partials; ++p) v += load_as_float(proj, proj_dt, p * partial_stride + in_row + col);
+    return v;
+  };
+
+  // query heads 0..nq-1, then key heads: one wave a head, four elements a lane (dk <= 256)
+  for (int head = wave; head < nq + nkv; head += kThreads / kWave) {
+    float x[4], ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = lane + 64 * u;
+      x[u] = e < dk ? value(head * dk + e) : 0.f;
+      ss += x[u] * x[u];
+    }
+    float inv = 1.f;
+    if (unit_norm) inv = 1.f / sqrtf(wave_sum(ss) / static_cast<float>(dk) + eps);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = lane + 64 * u;
+      if (e >= dk) continue;
+      if (head < nq) {
+        store_from_float(q_out, q_dt, (static_cast<size_t>(n) * nq + head) * dk + e, x[u] * inv);
+      } else if (slot >= 0) {
+        k_cache[((static_cast<size_t>(page) * nkv + (head - nq)) * page_size + off) * dk + e] = from_float<TC>(x[u] * inv);
+      }
+    }
+  }
+  const int v0 = (nq + nkv) * dk;
+  if (slot >= 0)
+    for (int i = tid; i < nkv * dv; i += kThreads) {
+      const int g = i / dv, e = i % dv;
+      v_cache[((static_cast<size_t>(page) * nkv + g) * page_size + off) * dv + e] = from_float<TC>(value(v0 + i));
+    }
+  if (gated)
+    for (int h = tid; h < nq; h += kThreads) gate_out[static_cast<size_t>(n) * nq + h] = 1.f / (1.f + expf(-value(v0 + nkv * dv + h)));
+}
+
+// ---------------------------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+constexpr int kKeys = 32;
+constexpr int kTileMaxKeyHead = 128;  // the queries of a block's four heads lie in LDS
+
+__device__ inline float shaped_score(float raw, float scale, float cap, const float* bias_row, int dist, int far) {
+  float s = raw * scale;
+  if (cap > 0.f) s = cap * tanhf(s / cap);
+  if (bias_row) s += bias_row[min(dist, far)];
+  return s;
+}
+
+// NV: the value head's size in tiles of 32 (the rest of the last tile is zeros); the key head's
+// size is a run-time number of up to 128, padded to a multiple of 32 in LDS. Layout as in attention_f32_mfma.hip:
+// the transposed problem, S^T[key, token] and O^T[d, token], so that a lane's sixteen scores are
+// the operands of the second product as they are.
+template <typename T, int NV>
+__global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
+    const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, T* __restrict__ out,
+    int out_ld, const float* __restrict__ gate, float out_scale, const int* __restrict__ tiles,
+    const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
+    int table_stride, int nq, int nkv, int dk, int dkp, int dv, int page_size, float scale, float cap,
+    const float* __restrict__ bias, int far, int window, int keep_first) {
+  extern __shared__ float lds[];
+  float* Ks = lds;                              // [kKeys][dkp + 1]
+  float* Qs = Ks + kKeys * (dkp + 1);           // [4 waves][32 tokens][dkp + 1]
+  float* Vt = Qs + 4 * 32 * (dkp + 1);          // [32 NV][kKeys + 1]
+  __shared__ int page_s[kKeys];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, h = lane >> 5, c = lane & 31;
+  const int n_rep = nq / nkv, hgroups = (n_rep + 3) / 4;
+  const int kvh = blockIdx.y / hgroups, hin = (blockIdx.y % hgroups) * 4 + wave;
+  const bool active = hin < n_rep;  // a wave without a head still helps loading
+  const int head = kvh * n_rep + (active ? hin : 0);
+  const int t0 = tiles[2 * blockIdx.x], ntok = tiles[2 * blockIdx.x + 1];
+  if (ntok <= 0) return;
+  const int pos0 = positions[t0];
+  const int* table = block_table + static_cast<size_t>(seq_of_token[t0]) * table_stride;
+  const int ldk = dkp + 1;
+
+  const bool live = active && c < ntok;
+  const int hi = c < ntok ? pos0 + c : pos0;
+  const int lo = window > 0 ? max(0, hi - window + 1) : 0;
+  const int keep = window > 0 ? keep_first : 0;
+  const float* bias_row = bias ? bias + static_cast<size_t>(head) * (far + 1) : nullptr;
+  {  // this wave's queries: Qs[wave][token][d], zeros where there is no token or no element
+    float* mine = Qs + wave * 32 * ldk;
+    for (int i = lane; i < 32 * dkp; i += 64) {
+      const int t = i / dkp, d = i % dkp;
+      mine[t * ldk + d] = active && t < ntok && d < dk ? to_float(q[(static_cast<size_t>(t0 + t) * nq + head) * dk + d]) : 0.f;
+    }
+  }
+  const float* myq = Qs + wave * 32 * ldk + c * ldk;
+  f32x16 o[NV];
+#pragma unroll
+  for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[dt][i] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  // the chunks that hold the kept first tokens which the window has passed, then the window's
+  const int lo_all = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int hi_all = pos0 + ntok - 1;
+  const int kept_end = min(keep, lo_all);                        // keys 0 .. kept_end - 1 lie before every window
+  const int n_first = kept_end > 0 ? (kept_end - 1) / kKeys + 1 : 0;
+  const int chunk_b = max(lo_all / kKeys, n_first);
+  const int n_chunks = n_first + (hi_all / kKeys - chunk_b + 1);
+  for (int it = 0; it < n_chunks; ++it) {
+    const int chunk = it < n_first ? it : chunk_b + (it - n_first);
+    const int key0 = chunk * kKeys;
+    __syncthreads();  // the previous chunk has been read by every wave (and the queries are written)
+    if (tid < kKeys) {
+      const int key = key0 + tid, entry = key / page_size;
+      page_s[tid] = key <= hi_all && entry < table_stride ? table[entry] : -1;
+    }
+    __syncthreads();
+    for (int i = tid; i < kKeys * dkp; i += kThreads) {
+      const int key = i / dkp, d = i % dkp, page = page_s[key];
+      float v = 0.f;
+      if (page >= 0 && d < dk)
+        v = to_float(k_cache[((static_cast<size_t>(page) * nkv + kvh) * page_size + (key0 + key) % page_size) * dk + d]);
+      Ks[key * ldk + d] = v;
+    }
+    for (int i = tid; i < kKeys * 32 * NV; i += kThreads) {
+      const int key = i / (32 * NV), d = i % (32 * NV), page = page_s[key];
+      float v = 0.f;
+      if (page >= 0 && d < dv)
+        v = to_float(v_cache[((static_cast<size_t>(page) * nkv + kvh) * page_size + (key0 + key) % page_size) * dv + d]);
+      Vt[d * (kKeys + 1) + key] = v;
+    }
+    __syncthreads();
+    if (!active) continue;
+
+    f32x16 s;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+    const float* krow = Ks + c * ldk;
+    for (int st = 0; st < dkp / 2; ++st)
+      s = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[2 * st + h], myq[2 * st + h], s, 0, 0, 0);
+
+    // element i of s: key key0 + 8 (i / 4) + 4 h + i % 4, token c
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int kk = 8 * (i >> 2) + 4 * h + (i & 3), key = key0 + kk;
+      const bool seen = key <= hi && (key >= lo || key < keep) && page_s[kk] >= 0;
+      s[i] = seen ? shaped_score(s[i], scale, cap, bias_row, hi - key, far) : -INFINITY;
+      mx = fmaxf(mx, s[i]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = expf(m - m_use);
+    m = m_new;
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      s[i] = expf(s[i] - m_use);
+      sum += s[i];
+    }
+    l = l * alpha + sum;
+#pragma unroll
+    for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+#pragma unroll
+    for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+      for (int st = 0; st < 16; ++st)
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(Vt[(32 * dt + c) * (kKeys + 1) + 8 * (st >> 2) + 4 * h + (st & 3)],
+                                                     s[st], o[dt], 0, 0, 0);
+  }
+
+  if (!active) return;
+  l += __shfl_xor(l, 32, 64);
+  if (!live) return;
+  float f = (l > 0.f ? 1.f / l : 0.f) * out_scale;
+  if (gate) f *= gate[static_cast<size_t>(t0 + c) * nq + head];
+  T* dst = out + static_cast<size_t>(t0 + c) * out_ld + head * dv;
+#pragma unroll
+  for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int d = 32 * dt + 8 * (i >> 2) + 4 * h + (i & 3);
+      if (d < dv) dst[d] = from_float<T>(o[dt][i] * f);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+constexpr int kSpan = 128;
+constexpr int kMaxHead = 256;
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void attn_biased_single_kernel(
+    const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, T* __restrict__ out,
+    int out_ld, const float* __restrict__ gate, float out_scale, const int* __restrict__ tokens,
+    const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
+    int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale, float cap,
+    const float* __restrict__ bias, int far, int window, int keep_first) {
+  __shared__ float qs[kMaxHead];
+  __shared__ float sc[kSpan];
+  __shared__ float accs[kThreads];
+  __shared__ float scratch[16];
+  const int n = tokens ? tokens[blockIdx.x] : blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int kvh = h / (nq / nkv);
+  const int pos = positions[n];
+  const int* table = block_table + static_cast<size_t>(seq_of_token[n]) * table_stride;
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int kept_end = window > 0 ? min(keep_first, lo) : 0;  // keys 0 .. kept_end - 1, then lo .. pos
+  const float* bias_row = bias ? bias + static_cast<size_t>(h) * (far + 1) : nullptr;
+  for (int d = tid; d < dk; d += kThreads) qs[d] = to_float(q[(static_cast<size_t>(n) * nq + h) * dk + d]);
+  __syncthreads();
+
+  const int groups = kThreads / dv;  // >= 1: dv <= 256
+  const int g = tid / dv, d = tid % dv;
+  const bool active = g < groups;
+  float m = -INFINITY, l = 0.f, acc = 0.f;
+  const int spans_first = (kept_end + kSpan - 1) / kSpan, spans_all = spans_first + (pos - lo) / kSpan + 1;
+  for (int span = 0; span < spans_all; ++span) {
+    const int base = span < spans_first ? span * kSpan : lo + (span - spans_first) * kSpan;
+    const int cnt = min(kSpan, (span < spans_first ? kept_end : pos + 1) - base);
+    float lmax = -INFINITY;
+    for (int j = tid; j < cnt; j += kThreads) {
+      const int key = base + j;
+      const int page = table[key / page_size], off = key % page_size;
+      float s = -INFINITY;
+      if (page >= 0) {
+        const T* kp = k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + off) * dk;
+        s = 0.f;
+        for (int e = 0; e < dk; ++e) s = fmaf(qs[e], to_float(kp[e]), s);
+        s = shaped_score(s, scale, cap, bias_row, pos - key, far);
+      }
+      sc[j] = s;
+      lmax = fmaxf(lmax, s);
+    }
+    const float m_new = fmaxf(m, block_max(lmax, scratch));
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = expf(m - m_use);
+    m = m_new;
+    float lsum = 0.f;
+    for (int j = tid; j < cnt; j += kThreads) {
+      const float p = expf(sc[j] - m_use);
+      sc[j] = p;
+      lsum += p;
+    }
+    l = l * alpha + block_sum(lsum, scratch);  // its barriers publish sc[]
+    acc *= alpha;
+    if (active)
+      for (int j = g; j < cnt; j += groups) {
+        const int key = base + j;
+        const int page = table[key / page_size], off = key % page_size;
+        if (page < 0) continue;
+        acc = fmaf(sc[j], to_float(v_cache[((static_cast<size_t>(page) * nkv + kvh) * page_size + off) * dv + d]), acc);
+      }
+    __syncthreads();  // sc[] is read; the next span may write it
+  }
+  accs[tid] = active ? acc : 0.f;
+  __syncthreads();
+  if (tid < dv) {
+    float total = 0.f;
+    for (int gg = 0; gg < groups; ++gg) total += accs[gg * dv + tid];
+    float f = (l > 0.f ? 1.f / l : 0.f) * out_scale;
+    if (gate) f *= gate[static_cast<size_t>(n) * nq + h];
+    out[static_cast<size_t>(n) * out_ld + h * dv + tid] = from_float<T>(total * f);
+  }
+}
+
+int check_geometry(const char* what, int nq, int nkv, int dk, int dv, int page_size) {
+  PYRE_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "%s: %d query heads do not divide over %d key/value heads", what, nq, nkv);
+  PYRE_REQUIRE(dk > 0 && dk <= kMaxHead && dv > 0 && dv <= kMaxHead, "%s: head sizes %d / %d are outside 1..%d", what, dk, dv, kMaxHead);
+  PYRE_REQUIRE(page_size > 0 && nq <= 65535, "%s: bad page size or too many heads", what);
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int pyre_unit_qkv_write(const void* proj, int proj_dt, int n_partials, long partial_stride, int ld, int col0,
+                                   void* q_out, int q_dt, void* k_cache, void* v_cache, int cache_dt, float* gate_out,
+                                   const int* slots, int n, int nq, int nkv, int dk, int dv, int page_size,
+                                   int unit_norm, float eps, int write_kv, hipStream_t stream) {
+  if (check_geometry("unit_qkv_write", nq, nkv, dk, dv, page_size)) return 1;
+  PYRE_REQUIRE(known_dtype(proj_dt) && known_dtype(q_dt) && known_dtype(cache_dt) && n_partials >= 1, "unit_qkv_write: bad dtypes");
+  PYRE_REQUIRE(!write_kv || (k_cache && v_cache && slots), "unit_qkv_write: a cache write needs caches and slots");
+  PYRE_REQUIRE(!unit_norm || eps > 0.f, "unit_qkv_write: eps must be positive");
+  if (n <= 0) return 0;
+  PYRE_DISPATCH(cache_dt, TC,
+      hipLaunchKernelGGL(unit_qkv_write_kernel<TC>, dim3(n), dim3(kThreads), 0, stream, proj, proj_dt, n_partials,
+                         static_cast<size_t>(partial_stride), ld, col0, q_out, q_dt, static_cast<TC*>(k_cache),
+                         static_cast<TC*>(v_cache), gate_out, slots, nq, nkv, dk, dv, page_size, unit_norm, eps,
+                         gate_out ? 1 : 0, write_kv));
+  return check_launch("unit_qkv_write");
+}
+
+extern "C" int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int dt, const void* k_cache, const void* v_cache,
+                                     const float* gate, float out_scale, const int* tiles, int n_tiles,
+                                     const int* positions, const int* seq_of_token, const int* block_table,
+                                     int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale,
+                                     float cap, const float* bias, int far, int window, int keep_first,
+                                     hipStream_t stream) {
+  if (check_geometry("attn_biased_tile", nq, nkv, dk, dv, page_size)) return 1;
+  PYRE_REQUIRE(known_dtype(dt) && table_stride > 0 && window >= 0 && keep_first >= 0 && far >= 0, "attn_biased_tile: bad arguments");
+  PYRE_REQUIRE(dk <= kTileMaxKeyHead, "attn_biased_tile: key heads of %d elements are more than %d", dk, kTileMaxKeyHead);
+  if (n_tiles <= 0) return 0;
+  const int hgroups = (nq / nkv + 3) / 4;
+  PYRE_REQUIRE(nkv * hgroups <= 65535, "attn_biased_tile: grid too large");
+  const int dkp = (dk + 31) / 32 * 32, nv = (dv + 31) / 32;
+  const int nvp = nv <= 1 ? 1 : nv <= 2 ? 2 : nv <= 4 ? 4 : 8;
+  const size_t lds = sizeof(float) * (static_cast<size_t>(kKeys + 4 * 32) * (dkp + 1) + 32 * nvp * (kKeys + 1));
+  const dim3 grid(n_tiles, nkv * hgroups);
+#define PYRE_TILE(T, NV)                                                                                             \
+  do {                                                                                                               \
+    static size_t raised = 64 * 1024;                                                                                \
+    if (lds > raised) {                                                                                              \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_biased_tile_kernel<T, NV>),                        \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess)      \
+        return fail("attn_biased_tile: the device refuses %zu bytes of LDS", lds);                                   \
+      raised = lds;                                                                                                  \
+    }                                                                                                                \
+    hipLaunchKernelGGL((attn_biased_tile_kernel<T, NV>), grid, dim3(kThreads), lds, stream, static_cast<const T*>(q), \
+                       static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), static_cast<T*>(out), out_ld, \
+                       gate, out_scale, tiles, positions, seq_of_token, block_table, table_stride, nq, nkv, dk, dkp,  \
+                       dv, page_size, scale, cap, bias, far, window, keep_first);                                    \
+  } while (0)
+#define PYRE_TILE_NV(T)                \
+  switch (nvp) {                       \
+    case 1: PYRE_TILE(T, 1); break;    \
+    case 2: PYRE_TILE(T, 2); break;    \
+    case 4: PYRE_TILE(T, 4); break;    \
+    default: PYRE_TILE(T, 8); break;   \
+  }
+  if (dt == kF32) { PYRE_TILE_NV(float) } else { PYRE_TILE_NV(bf16) }
+#undef PYRE_TILE_NV
+#undef PYRE_TILE
+  return check_launch("attn_biased_tile");
+}
+
+extern "C" int pyre_attn_biased_single(const void* q, void* out, int out_ld, int dt, const void* k_cache,
+                                       const void* v_cache, const float* gate, float out_scale, const int* tokens,
+                                       int n, const int* positions, const int* seq_of_token, const int* block_table,
+                                       int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale,
+                                       float cap, const float* bias, int far, int window, int keep_first,
+                                       hipStream_t stream) {
+  if (check_geometry("attn_biased_single", nq, nkv, dk, dv, page_size)) return 1;
+  PYRE_REQUIRE(known_dtype(dt) && table_stride > 0 && window >= 0 && keep_first >= 0 && far >= 0, "attn_biased_single: bad arguments");
+  if (n <= 0) return 0;
+  PYRE_DISPATCH(dt, T,
+      hipLaunchKernelGGL(attn_biased_single_kernel<T>, dim3(n, nq), dim3(kThreads), 0, stream, static_cast<const T*>(q),
+                         static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), static_cast<T*>(out), out_ld,
+                         gate, out_scale, tokens, positions, seq_of_token, block_table, table_stride, nq, nkv, dk, dv,
+                         page_size, scale, cap, bias, far, window, keep_first));
+  return check_launch("attn_biased_single");
+}

@@ -1,0 +1,168 @@
+// Layer norm around the float32 residual stream, for blocks that norm a sublayer's result
+// before it is added ("sandwich" blocks), a gated feed-forward activation with clipped inputs,
+// and a scaling of float32 rows. All arithmetic float32.
+//
+//   d      = sum of the pending partial sums (+ bias)
+//   y      = post ? LN(d; post_eps) * post_gain * post_scale : d       (the sublayer's own norm and layer scale)
+//   resid += y
+//   out    = LN(resid; eps) * gain
+//   LN(x; e) = (x - mean(x)) / sqrt(mean((x - mean(x))^2) + e)
+//
+// One block per row; a thread keeps its elements in registers (every 256th), so the row is read
+// once. Mean and variance are two separate sums, the variance over the deviations from the mean.
+// With `rows` only the listed rows are normed, into out[0 .. n), and resid is left as it was.
+#include "pyre_api.h"
+#include "pyre_common.h"
+
+using namespace pyre;
+
+namespace {
+
+constexpr int kThreads = 256;
+
+template <int ITEMS>
+__global__ __launch_bounds__(kThreads) void add_layernorm_kernel(
+    float* __restrict__ resid, const void* __restrict__ delta, int delta_dt, int n_partials, size_t partial_stride,
+    const void* __restrict__ bias, int bias_dt, const void* __restrict__ post_gain, int post_gain_dt,
+    const void* __restrict__ post_scale, int post_scale_dt, float post_eps, const void* __restrict__ gain,
+    int gain_dt, void* __restrict__ out, int out_dt, const int* __restrict__ rows, int hidden, float eps) {
+  __shared__ float scratch[16];
+  const int r_out = blockIdx.x, r_in = rows ? rows[r_out] : r_out, tid = threadIdx.x;
+  const size_t row = static_cast<size_t>(r_in) * hidden;
+  const float inv_n = 1.f / static_cast<float>(hidden);
+  float v[ITEMS];
+
+  // mean and 1 / sqrt(variance + e) of the row held in v
+  auto stats = [&](float e, float& mean, float& inv) {
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k)
+      if (tid + k * kThreads < hidden) s += v[k];
+    mean = block_sum(s, scratch) * inv_n;
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k)
+      if (tid + k * kThreads < hidden) ss += (v[k] - mean) * (v[k] - mean);
+    inv = 1.f / sqrtf(block_sum(ss, scratch) * inv_n + e);
+  };
+
+  if (delta) {
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+      const int i = tid + k * kThreads;
+      float d = 0.f;
+      if (i < hidden) {
+        for (int p = 0; p < n_partials; ++p) d += load_as_float(delta, delta_dt, p * partial_stride + row + i);
+        if (bias) d += load_as_float(bias, bias_dt, i);
+      }
+      v[k] = d;
+    }
+    if (post_gain) {
+      float mean, inv;
+      stats(post_eps, mean, inv);
+#pragma unroll
+      for (int k = 0; k < ITEMS; ++k) {
+        const int i = tid + k * kThreads;
+        if (i < hidden) {
+          float y = (v[k] - mean) * inv * load_as_float(post_gain, post_gain_dt, i);
+          if (post_scale) y *= load_as_float(post_scale, post_scale_dt, i);
+          v[k] = y;
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+      const int i = tid + k * kThreads;
+      if (i < hidden) {
+        v[k] += resid[row + i];
+        if (!rows) resid[row + i] = v[k];
+      }
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+      const int i = tid + k * kThreads;
+      v[k] = i < hidden ? resid[row + i] : 0.f;
+    }
+  }
+  float mean, inv;
+  stats(eps, mean, inv);
+  const size_t orow = static_cast<size_t>(r_out) * hidden;
+#pragma unroll
+  for (int k = 0; k < ITEMS; ++k) {
+    const int i = tid + k * kThreads;
+    if (i < hidden) store_from_float(out, out_dt, orow + i, (v[k] - mean) * inv * load_as_float(gain, gain_dt, i));
+  }
+}
+
+// act[n, i] = g * sigmoid(slope * g) * (u + 1), g = min(gate[n, i], limit), u = clamp(up[n, i], -limit, limit);
+// gate = gu[:, :I], up = gu[:, I:], the partial sums added first. limit <= 0: no clipping.
+__global__ void clipped_glu_kernel(const void* __restrict__ gu, int gu_dt, int n_partials, size_t partial_stride,
+                                   void* __restrict__ out, int out_dt, size_t total, int inter, float limit,
+                                   float slope) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t n = i / inter, c = i % inter;
+  const size_t gi = n * 2 * inter + c, ui = gi + inter;
+  float g = 0.f, u = 0.f;
+  for (int p = 0; p < n_partials; ++p) {
+    g += load_as_float(gu, gu_dt, p * partial_stride + gi);
+    u += load_as_float(gu, gu_dt, p * partial_stride + ui);
+  }
+  if (limit > 0.f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+  }
+  store_from_float(out, out_dt, i, g / (1.f + expf(-slope * g)) * (u + 1.f));
+}
+
+__global__ void scale_kernel(float* __restrict__ x, size_t total, float s) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < total) x[i] *= s;
+}
+
+}  // namespace
+
+extern "C" int pyre_add_layernorm(float* resid, const void* delta, int delta_dt, int n_partials, long partial_stride,
+                                  const void* bias, int bias_dt, const void* post_gain, int post_gain_dt,
+                                  const void* post_scale, int post_scale_dt, float post_eps, const void* gain,
+                                  int gain_dt, void* out, int out_dt, const int* rows, int n, int hidden, float eps,
+                                  hipStream_t stream) {
+  PYRE_REQUIRE(known_dtype(gain_dt) && known_dtype(out_dt), "add_layernorm: unknown dtype");
+  PYRE_REQUIRE(!delta || (known_dtype(delta_dt) && n_partials >= 1), "add_layernorm: bad delta (dtype %d, partials %d)",
+               delta_dt, n_partials);
+  PYRE_REQUIRE(!bias || known_dtype(bias_dt), "add_layernorm: unknown bias dtype");
+  PYRE_REQUIRE(!post_gain || (delta && known_dtype(post_gain_dt) && post_eps > 0.f),
+               "add_layernorm: a norm of the pending term needs the term, a gain and a positive eps");
+  PYRE_REQUIRE(!post_scale || (post_gain && known_dtype(post_scale_dt)), "add_layernorm: a layer scale without its norm");
+  PYRE_REQUIRE(n >= 0 && hidden > 0 && eps > 0.f, "add_layernorm: bad sizes n=%d hidden=%d", n, hidden);
+  PYRE_REQUIRE(hidden <= 64 * kThreads, "add_layernorm: rows of %d elements are more than %d", hidden, 64 * kThreads);
+  if (n == 0) return 0;
+#define PYRE_LN(ITEMS)                                                                                              \
+  hipLaunchKernelGGL(add_layernorm_kernel<ITEMS>, dim3(n), dim3(kThreads), 0, stream, resid, delta, delta_dt,       \
+                     n_partials, static_cast<size_t>(partial_stride), bias, bias_dt, post_gain, post_gain_dt,       \
+                     post_scale, post_scale_dt, post_eps, gain, gain_dt, out, out_dt, rows, hidden, eps)
+  if (hidden <= 2 * kThreads) PYRE_LN(2);
+  else if (hidden <= 8 * kThreads) PYRE_LN(8);
+  else if (hidden <= 32 * kThreads) PYRE_LN(32);
+  else PYRE_LN(64);
+#undef PYRE_LN
+  return check_launch("add_layernorm");
+}
+
+extern "C" int pyre_clipped_glu(const void* gu, int gu_dt, int n_partials, long partial_stride, void* out, int out_dt,
+                                int n, int inter, float limit, float slope, hipStream_t stream) {
+  PYRE_REQUIRE(known_dtype(gu_dt) && known_dtype(out_dt), "clipped_glu: unknown dtype");
+  PYRE_REQUIRE(n_partials >= 1 && inter > 0, "clipped_glu: bad sizes");
+  if (n <= 0) return 0;
+  const size_t total = static_cast<size_t>(n) * inter;
+  hipLaunchKernelGGL(clipped_glu_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, gu, gu_dt, n_partials,
+                     static_cast<size_t>(partial_stride), out, out_dt, total, inter, limit, slope);
+  return check_launch("clipped_glu");
+}
+
+extern "C" int pyre_scale(float* x, long total, float s, hipStream_t stream) {
+  if (total <= 0) return 0;
+  hipLaunchKernelGGL(scale_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, x, static_cast<size_t>(total), s);
+  return check_launch("scale");
+}

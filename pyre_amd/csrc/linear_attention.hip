@@ -1,0 +1,168 @@
+// Gated linear attention: per head a float32 matrix state S [dk, dv] that every token decays
+// row by row and adds an outer product to, read by the token's query:
+//
+//   S_t = diag(a_t) S_(t-1) + k_t v_t^T,      o_t = qscale * S_t^T q_t,      a_t = exp(ld_t), ld_t <= 0
+//
+// gla_prepare  finishes the input product of a step (partial sums) into float32 rows
+//              [q | k | ld | v | g] and makes the logarithm of the decay from a low-rank product:
+//              z = A2 (A1 h) + b,  ld = log(sigmoid(z)) / tau  (so that a = sigmoid(z)^(1/tau)).
+// gla_scan     walks the tokens of every request of the step in their order from the state that
+//              earlier steps left in the request's slot, and leaves the new state there.
+// gla_finish   divides every head's output by its root mean square, times a gain over dv that the
+//              heads share, times silu(g) and a scale; writes the rows that the output product reads.
+//
+// Decays, their logarithms, the state and the unit norm are float32 whatever the model's type.
+#include "pyre_api.h"
+#include "pyre_common.h"
+
+using namespace pyre;
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaxRank = 512;
+
+__global__ __launch_bounds__(kThreads) void gla_prepare_kernel(
+    const void* __restrict__ proj, int proj_dt, int n_partials, size_t partial_stride, int ld, int col0,
+    const void* __restrict__ a2, int a2_dt, const void* __restrict__ a2_bias, int bias_dt, float inv_tau,
+    float* __restrict__ x, int heads, int dk, int dv, int rank) {
+  __shared__ float a1s[kMaxRank];
+  const int n = blockIdx.x, tid = threadIdx.x;
+  const size_t in_row = static_cast<size_t>(n) * ld + col0;
+  const int hk = heads * dk, hv = heads * dv, width = 3 * hk + 2 * hv;
+  float* xr = x + static_cast<size_t>(n) * width;
+  auto value = [&](int col) {
+    float v = 0.f;
+    for (int p = 0; p < n_partials; ++p) v += load_as_float(proj, proj_dt, p * partial_stride + in_row + col);
+    return v;
+  };
+  // the product's columns: q, k (hk each), v, g (hv each), the low-rank input (rank)
+  for (int r = tid; r < rank; r += kThreads) a1s[r] = value(2 * hk + 2 * hv + r);
+  for (int i = tid; i < 2 * hk; i += kThreads) xr[i] = value(i);
+  for (int i = tid; i < 2 * hv; i += kThreads) xr[3 * hk + i] = value(2 * hk + i);
+  __syncthreads();
+  for (int c = tid; c < hk; c += kThreads) {
+    float z = 0.f;
+    for (int r = 0; r < rank; ++r) z = fmaf(load_as_float(a2, a2_dt, static_cast<size_t>(c) * rank + r), a1s[r], z);
+    if (a2_bias) z += load_as_float(a2_bias, bias_dt, c);
+    // log(sigmoid(z)) without overflow on either side
+    const float ls = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
+    xr[2 * hk + c] = ls * inv_tau;
+  }
+}
+
+// A block: one request, one head, 64 columns of the state (a lane a column); wave w keeps the rows
+// w, w + 4, ... in registers, DR of them. A token's four partial outputs are joined through LDS.
+template <int DR>
+__global__ __launch_bounds__(kThreads) void gla_scan_kernel(
+    const float* __restrict__ x, float* __restrict__ state, float* __restrict__ o, const int* __restrict__ q_start,
+    const int* __restrict__ state_slots, int heads, int dk, int dv, float qscale) {
+  __shared__ float red[2][4][kWave];
+  const int s = blockIdx.x, hd = blockIdx.y, tid = threadIdx.x, w = tid >> 6, lane = tid & 63;
+  const int col = blockIdx.z * kWave + lane;
+  const bool has_col = col < dv;
+  const int t_begin = q_start[s], t_end = q_start[s + 1];
+  const int hk = heads * dk, hv = heads * dv, width = 3 * hk + 2 * hv;
+  float* st = state + (static_cast<size_t>(state_slots[s]) * heads + hd) * dk * dv;
+  float S[DR];
+#pragma unroll
+  for (int r = 0; r < DR; ++r) {
+    const int row = w + 4 * r;
+    S[r] = has_col && row < dk ? st[static_cast<size_t>(row) * dv + col] : 0.f;
+  }
+  for (int t = t_begin; t < t_end; ++t) {
+    const float* xr = x + static_cast<size_t>(t) * width;
+    const float* qr = xr + hd * dk;
+    const float* kr = qr + hk;
+    const float* lr = kr + hk;
+    const float v = has_col ? xr[3 * hk + hd * dv + col] : 0.f;
+    float part = 0.f;
+#pragma unroll
+    for (int r = 0; r < DR; ++r) {
+      const int row = w + 4 * r;
+      if (row < dk) {
+        S[r] = expf(lr[row]) * S[r] + kr[row] * v;
+        part = fmaf(S[r], qr[row], part);
+      }
+    }
+    const int buf = (t - t_begin) & 1;
+    red[buf][w][lane] = part;
+    __syncthreads();
+    if (w == 0 && has_col)
+      o[static_cast<size_t>(t) * hv + hd * dv + col] =
+          (((red[buf][0][lane] + red[buf][1][lane]) + red[buf][2][lane]) + red[buf][3][lane]) * qscale;
+  }
+#pragma unroll
+  for (int r = 0; r < DR; ++r) {
+    const int row = w + 4 * r;
+    if (has_col && row < dk) st[static_cast<size_t>(row) * dv + col] = S[r];
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void gla_finish_kernel(
+    const float* __restrict__ o, const float* __restrict__ x, const void* __restrict__ gain, int gain_dt, float eps,
+    float out_scale, void* __restrict__ out, int out_dt, int out_ld, int heads, int dk, int dv) {
+  const int n = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int hk = heads * dk, hv = heads * dv, width = 3 * hk + 2 * hv;
+  const float* g = x + static_cast<size_t>(n) * width + 3 * hk + hv;
+  for (int hd = wave; hd < heads; hd += kThreads / kWave) {
+    float v[4], ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = lane + 64 * u;
+      v[u] = e < dv ? o[static_cast<size_t>(n) * hv + hd * dv + e] : 0.f;
+      ss += v[u] * v[u];
+    }
+    const float inv = 1.f / sqrtf(wave_sum(ss) / static_cast<float>(dv) + eps);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = lane + 64 * u;
+      if (e >= dv) continue;
+      const float gg = g[hd * dv + e];
+      const float y = v[u] * inv * load_as_float(gain, gain_dt, e) * (gg / (1.f + expf(-gg))) * out_scale;
+      store_from_float(out, out_dt, static_cast<size_t>(n) * out_ld + hd * dv + e, y);
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int pyre_gla_prepare(const void* proj, int proj_dt, int n_partials, long partial_stride, int ld, int col0,
+                                const void* a2, int a2_dt, const void* a2_bias, int bias_dt, float tau, float* x,
+                                int n, int heads, int dk, int dv, int rank, hipStream_t stream) {
+  PYRE_REQUIRE(known_dtype(proj_dt) && known_dtype(a2_dt) && (!a2_bias || known_dtype(bias_dt)) && n_partials >= 1,
+               "gla_prepare: bad dtypes");
+  PYRE_REQUIRE(heads > 0 && dk > 0 && dv > 0 && rank > 0 && rank <= kMaxRank, "gla_prepare: bad sizes (rank %d of at most %d)", rank, kMaxRank);
+  PYRE_REQUIRE(tau > 0.f, "gla_prepare: tau must be positive");
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(gla_prepare_kernel, dim3(n), dim3(kThreads), 0, stream, proj, proj_dt, n_partials,
+                     static_cast<size_t>(partial_stride), ld, col0, a2, a2_dt, a2_bias, bias_dt, 1.f / tau, x, heads, dk,
+                     dv, rank);
+  return check_launch("gla_prepare");
+}
+
+extern "C" int pyre_gla_scan(const float* x, float* state, float* o, const int* q_start, const int* state_slots,
+                             int n_seqs, int heads, int dk, int dv, float qscale, hipStream_t stream) {
+  PYRE_REQUIRE(heads > 0 && heads <= 65535 && dk > 0 && dk <= 256 && dv > 0, "gla_scan: heads %d, sizes %d / %d are not taken", heads, dk, dv);
+  if (n_seqs <= 0) return 0;
+  const dim3 grid(n_seqs, heads, (dv + kWave - 1) / kWave);
+#define PYRE_SCAN(DR)                                                                                            \
+  hipLaunchKernelGGL(gla_scan_kernel<DR>, grid, dim3(kThreads), 0, stream, x, state, o, q_start, state_slots, heads, \
+                     dk, dv, qscale)
+  if (dk <= 32) PYRE_SCAN(8);
+  else if (dk <= 64) PYRE_SCAN(16);
+  else if (dk <= 128) PYRE_SCAN(32);
+  else PYRE_SCAN(64);
+#undef PYRE_SCAN
+  return check_launch("gla_scan");
+}
+
+extern "C" int pyre_gla_finish(const float* o, const float* x, const void* gain, int gain_dt, float eps, float out_scale,
+                               void* out, int out_dt, int out_ld, int n, int heads, int dk, int dv, hipStream_t stream) {
+  PYRE_REQUIRE(known_dtype(gain_dt) && known_dtype(out_dt), "gla_finish: bad dtypes");
+  PYRE_REQUIRE(heads > 0 && dk > 0 && dv > 0 && dv <= 256 && eps > 0.f, "gla_finish: sizes %d / %d are not taken", dk, dv);
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(gla_finish_kernel, dim3(n), dim3(kThreads), 0, stream, o, x, gain, gain_dt, eps, out_scale, out,
+                     out_dt, out_ld, heads, dk, dv);
+  return check_launch("gla_finish");
+}

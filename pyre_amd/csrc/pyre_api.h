@@ -208,4 +208,53 @@ int pyre_feed_tokens(int* tokens, const int* src, const int* ids, int n, hipStre
 int pyre_sample(const float* logits, long row_stride, const float* temperature,
                 const float* uniform, int* out, int m, int vocab, hipStream_t stream);
 
+// ---- layer norm around the residual stream, clipped gated activation, scaling (layernorm.hip) ----
+// resid += y, out = LN(resid) * gain, where y is the pending term (partial sums, bias) or, with
+// post_gain, LN(term; post_eps) * post_gain (* post_scale). rows: only these rows, resid untouched.
+int pyre_add_layernorm(float* resid, const void* delta, int delta_dt, int n_partials, long partial_stride,
+                       const void* bias, int bias_dt, const void* post_gain, int post_gain_dt,
+                       const void* post_scale, int post_scale_dt, float post_eps, const void* gain,
+                       int gain_dt, void* out, int out_dt, const int* rows, int n, int hidden, float eps,
+                       hipStream_t stream);
+// out[n, i] = g sigmoid(slope g) (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit); gu = [gate | up].
+int pyre_clipped_glu(const void* gu, int gu_dt, int n_partials, long partial_stride, void* out, int out_dt,
+                     int n, int inter, float limit, float slope, hipStream_t stream);
+int pyre_scale(float* x, long total, float s, hipStream_t stream);
+
+// ---- attention with capped scores, a bias by distance and kept first tokens (attention_biased.hip) ----
+// proj columns from col0 on: nq query heads and nkv key heads of dk, nkv value heads of dv, then (gate_out
+// given) nq gates. Caches: k [pages, nkv, page, dk], v [pages, nkv, page, dv].
+int pyre_unit_qkv_write(const void* proj, int proj_dt, int n_partials, long partial_stride, int ld, int col0,
+                        void* q_out, int q_dt, void* k_cache, void* v_cache, int cache_dt, float* gate_out,
+                        const int* slots, int n, int nq, int nkv, int dk, int dv, int page_size,
+                        int unit_norm, float eps, int write_kv, hipStream_t stream);
+// tiles: [n_tiles][2] = (first token, count <= 32). bias: float32 [nq][far + 1] by distance, or null.
+// gate: float32 [tokens][nq] or null. out rows are out_ld elements apart; head h writes columns h dv ...
+int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int dt, const void* k_cache, const void* v_cache,
+                          const float* gate, float out_scale, const int* tiles, int n_tiles,
+                          const int* positions, const int* seq_of_token, const int* block_table,
+                          int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale,
+                          float cap, const float* bias, int far, int window, int keep_first,
+                          hipStream_t stream);
+// tokens: the n tokens of the flat batch to attend for (null: 0..n-1), a block per token and head.
+int pyre_attn_biased_single(const void* q, void* out, int out_ld, int dt, const void* k_cache,
+                            const void* v_cache, const float* gate, float out_scale, const int* tokens,
+                            int n, const int* positions, const int* seq_of_token, const int* block_table,
+                            int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale,
+                            float cap, const float* bias, int far, int window, int keep_first,
+                            hipStream_t stream);
+
+// ---- gated linear attention (linear_attention.hip) ----
+// proj columns from col0 on: q, k (heads dk each), v, g (heads dv each), the low-rank input (rank).
+// x: float32 [n][3 heads dk + 2 heads dv] = [q | k | log decay | v | g].
+int pyre_gla_prepare(const void* proj, int proj_dt, int n_partials, long partial_stride, int ld, int col0,
+                     const void* a2, int a2_dt, const void* a2_bias, int bias_dt, float tau, float* x,
+                     int n, int heads, int dk, int dv, int rank, hipStream_t stream);
+// state: float32 [slots][heads][dk][dv]; o: float32 [tokens][heads dv]; request s owns the tokens
+// q_start[s] .. q_start[s + 1] - 1 and the slot state_slots[s].
+int pyre_gla_scan(const float* x, float* state, float* o, const int* q_start, const int* state_slots,
+                  int n_seqs, int heads, int dk, int dv, float qscale, hipStream_t stream);
+int pyre_gla_finish(const float* o, const float* x, const void* gain, int gain_dt, float eps, float out_scale,
+                    void* out, int out_dt, int out_ld, int n, int heads, int dk, int dv, hipStream_t stream);
+
 }  // extern "C"

@@ -27,6 +27,8 @@ from pyre_amd.weights.loader import adopt_state, load_weights
 #: decode steps of up to this many requests are captured in HIP graphs, at these sizes
 GRAPH_ROW_BUCKETS = DECODE_ROW_BUCKETS
 GRAPH_MAX_ROWS = GRAPH_ROW_BUCKETS[-1]
+#: the longest request of a model that names no limit, when neither the caller nor the pool's size says
+DEFAULT_MAX_MODEL_LEN = 32768
 
 
 class Engine:
@@ -47,7 +49,8 @@ class Engine:
         spec = model.spec
         # The model's own limit is the default, not a bound: the reference reads
         # max_position_embeddings and never consults it (`pyre/config.py:60`).
-        self.max_model_len = ec.max_model_len or spec.max_positions
+        # A model without a limit of its own (max_positions 0) takes the pool's size, or a default.
+        self.max_model_len = ec.max_model_len or spec.max_positions or ec.max_cached_tokens or DEFAULT_MAX_MODEL_LEN
         with torch.cuda.device(self.device):
             self.runtime = Runtime(self.device, self.dtype, self.max_model_len)
         specs = model.cache_specs()

@@ -31,7 +31,7 @@ def main(argv: list[str] | None = None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page (a divisor of 64)")
-    ap.add_argument("--max-seqs", type=int, default=8, help="most requests that are live at a time")
+    ap.add_argument("--max-seqs", type=int, default=4, help="most requests that are live at a time")
     ap.add_argument("--poison", action="store_true",
                     help="debugging aid: freed cache pages and state slots are filled with NaN")
     ap.add_argument("--graphs", action="store_true",

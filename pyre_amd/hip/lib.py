@@ -11,7 +11,7 @@ from ctypes import c_float, c_int, c_long, c_void_p
 
 from pyre_amd.hip import build as _build
 
-ABI_VERSION = 19
+ABI_VERSION = 20
 
 
 class KernelError(RuntimeError):
@@ -53,6 +53,15 @@ _SIGNATURES = {
     "pyre_gemm_mid_silu_bf16": [P, L, P, L, P, I, I, I, P],
     "pyre_sample": [P, L, P, P, P, I, I, P],
     "pyre_feed_tokens": [P, P, P, I, P],
+    "pyre_add_layernorm": [P, P, I, I, L, P, I, P, I, P, I, F, P, I, P, I, P, I, I, F, P],
+    "pyre_clipped_glu": [P, I, I, L, P, I, I, I, F, F, P],
+    "pyre_scale": [P, L, F, P],
+    "pyre_unit_qkv_write": [P, I, I, L, I, I, P, I, P, P, I, P, P, I, I, I, I, I, I, I, F, I, P],
+    "pyre_attn_biased_tile": [P, P, I, I, P, P, P, F, P, I, P, P, P, I, I, I, I, I, I, F, F, P, I, I, I, P],
+    "pyre_attn_biased_single": [P, P, I, I, P, P, P, F, P, I, P, P, P, I, I, I, I, I, I, F, F, P, I, I, I, P],
+    "pyre_gla_prepare": [P, I, I, L, I, I, P, I, P, I, F, P, I, I, I, I, I, P],
+    "pyre_gla_scan": [P, P, P, P, P, I, I, I, I, F, P],
+    "pyre_gla_finish": [P, P, P, I, F, F, P, I, I, I, I, I, I, P],
 }
 
 _lib = None

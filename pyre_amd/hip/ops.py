@@ -64,6 +64,15 @@ def _ptr(t: torch.Tensor | None) -> int | None:
 
 
 @dataclass
+class PostNorm:
+    """The norm of a sublayer's own result: LN(term; eps) * gain (* scale), element by element."""
+
+    gain: torch.Tensor
+    eps: float
+    scale: torch.Tensor | None = None
+
+
+@dataclass
 class Partials:
     """What a matrix product hands to its consumer: ``S`` partial sums ``[S, M, N]``
     (``S`` = 1 unless the product was split along K) and a bias not yet added.
@@ -71,6 +80,9 @@ class Partials:
 
     data: torch.Tensor
     bias: torch.Tensor | None = None
+    #: a norm (and layer scale) that the term goes through before it is added: only a norm
+    #: that says so takes such a term (:func:`add_layernorm`)
+    post: "PostNorm | None" = None
 
     def __post_init__(self) -> None:
         if self.data.dim() != 3 or not self.data.is_contiguous():
@@ -132,11 +144,216 @@ def add_rmsnorm(resid: torch.Tensor, delta: Partials | None, gain: torch.Tensor,
     if delta is not None:
         if delta.rows < resid.shape[0]:
             raise KernelError("add_rmsnorm: delta has fewer rows than the residual")
+        if delta.post is not None:
+            raise KernelError("add_rmsnorm: a term that is to be normed before it is added is not taken")
         d = delta._args(hidden)
     else:
         d = (None, 0, 0, 0, None, 0)
     call("pyre_add_rmsnorm", resid.data_ptr(), *d, gain.data_ptr(), dtype_code(gain), out.data_ptr(),
          dtype_code(out), _ptr(rows), n, hidden, float(eps), _stream())
+
+
+def add_layernorm(resid: torch.Tensor, delta: Partials | None, gain: torch.Tensor, eps: float,
+                  out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
+    """resid += y; out = LN(resid) * gain, with LN(x) = (x - mean) / sqrt(var + eps) and y the
+    pending term (all partials, then bias), which goes through its own norm first if it carries one
+    (``delta.post``: y = LN(term; post.eps) * post.gain * post.scale).
+
+    With ``rows`` only those rows are normed, into ``out[0:len(rows)]``, and ``resid`` is left as it was.
+    """
+    _dev(resid, gain, out, rows)
+    hidden = resid.shape[-1]
+    if resid.dtype != torch.float32 or resid.dim() != 2:
+        raise KernelError("add_layernorm: the residual stream is float32 [N, H]")
+    n = resid.shape[0] if rows is None else rows.numel()
+    if out.shape[-1] != hidden or out.shape[0] < n or gain.numel() != hidden:
+        raise KernelError("add_layernorm: shapes of out / gain do not fit the residual")
+    _contig("resid", resid), _contig("out", out), _contig("gain", gain)
+    if rows is not None:
+        _i32("rows", rows)
+    post = (None, 0, None, 0, 0.0)
+    if delta is not None:
+        if delta.rows < resid.shape[0]:
+            raise KernelError("add_layernorm: delta has fewer rows than the residual")
+        d = delta._args(hidden)
+        if delta.post is not None:
+            pn = delta.post
+            _dev(pn.gain, pn.scale)
+            if pn.gain.numel() != hidden or (pn.scale is not None and pn.scale.numel() != hidden):
+                raise KernelError("add_layernorm: the pending term's gain / scale do not fit the residual")
+            _contig("post.gain", pn.gain)
+            if pn.scale is not None:
+                _contig("post.scale", pn.scale)
+            post = (pn.gain.data_ptr(), dtype_code(pn.gain), _ptr(pn.scale),
+                    dtype_code(pn.scale) if pn.scale is not None else 0, float(pn.eps))
+    else:
+        d = (None, 0, 0, 0, None, 0)
+    call("pyre_add_layernorm", resid.data_ptr(), *d, *post, gain.data_ptr(), dtype_code(gain), out.data_ptr(),
+         dtype_code(out), _ptr(rows), n, hidden, float(eps), _stream())
+
+
+def clipped_glu(gu: Partials, out: torch.Tensor, n: int, limit: float, slope: float) -> None:
+    """out[n, i] = g * sigmoid(slope * g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit),
+    gate = gu[:, :I], up = gu[:, I:] (``limit`` <= 0: no clipping)."""
+    _dev(gu.data, out)
+    inter = out.shape[-1]
+    if gu.width != 2 * inter or gu.rows < n or out.shape[0] < n:
+        raise KernelError("clipped_glu: gate/up buffer does not fit the output")
+    if gu.bias is not None:
+        raise KernelError("clipped_glu: a pending bias is not supported")
+    _contig("out", out)
+    call("pyre_clipped_glu", gu.data.data_ptr(), dtype_code(gu.data), gu.count, gu.stride, out.data_ptr(),
+         dtype_code(out), n, inter, float(limit), float(slope), _stream())
+
+
+def scale_(x: torch.Tensor, s: float) -> None:
+    """x *= s in place (contiguous float32)."""
+    _dev(x)
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelError("scale_: contiguous float32 expected")
+    call("pyre_scale", x.data_ptr(), x.numel(), float(s), _stream())
+
+
+def _proj_args(proj: Partials, col0: int, width: int):
+    if proj.bias is not None:
+        raise KernelError("a fused input product with a pending bias is not taken")
+    if col0 < 0 or col0 + width > proj.width:
+        raise KernelError(f"columns {col0}..{col0 + width} lie outside the product's {proj.width}")
+    return (proj.data.data_ptr(), dtype_code(proj.data), proj.count, proj.stride, proj.width, col0)
+
+
+def unit_qkv_write(proj: Partials, col0: int, q_out: torch.Tensor, k_cache: torch.Tensor | None,
+                   v_cache: torch.Tensor | None, gate_out: torch.Tensor | None, slots: torch.Tensor | None, n: int,
+                   nq: int, nkv: int, dk: int, dv: int, page_size: int, unit_norm: bool, eps: float) -> None:
+    """Finish a step's input product from column ``col0`` on (``nq`` query and ``nkv`` key heads of ``dk``,
+    ``nkv`` value heads of ``dv``, then ``nq`` gates if ``gate_out`` is given): queries and keys divided by
+    their root mean square over ``dk`` (``unit_norm``), queries to ``q_out [N, nq*dk]``, keys and values to
+    ``k_cache [pages, nkv, page, dk]`` / ``v_cache [pages, nkv, page, dv]`` at ``slots`` (-1: not stored),
+    sigmoid(gate) to float32 ``gate_out [N, nq]``."""
+    _dev(proj.data, q_out, k_cache, v_cache, gate_out, slots)
+    width = (nq + nkv) * dk + nkv * dv + (nq if gate_out is not None else 0)
+    args = _proj_args(proj, col0, width)
+    if proj.rows < n or q_out.numel() < n * nq * dk:
+        raise KernelError("unit_qkv_write: buffers are smaller than the batch")
+    _contig("q_out", q_out)
+    write = k_cache is not None
+    cache_dt = dtype_code(q_out)
+    if write:
+        if v_cache is None or slots is None:
+            raise KernelError("unit_qkv_write: k cache without v cache or slots")
+        _i32("slots", slots, n), _contig("k_cache", k_cache), _contig("v_cache", v_cache)
+        if tuple(k_cache.shape[1:]) != (nkv, page_size, dk) or tuple(v_cache.shape[1:]) != (nkv, page_size, dv) \
+                or k_cache.dtype != v_cache.dtype:
+            raise KernelError(f"unit_qkv_write: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} do not fit "
+                              f"nkv={nkv} page={page_size} dk={dk} dv={dv}")
+        cache_dt = dtype_code(k_cache)
+    if gate_out is not None and (gate_out.dtype != torch.float32 or gate_out.numel() < n * nq or not gate_out.is_contiguous()):
+        raise KernelError("unit_qkv_write: gates are contiguous float32 [N, nq]")
+    call("pyre_unit_qkv_write", *args, q_out.data_ptr(), dtype_code(q_out), _ptr(k_cache), _ptr(v_cache), cache_dt,
+         _ptr(gate_out), _ptr(slots), n, nq, nkv, dk, dv, page_size, int(bool(unit_norm)), float(eps),
+         1 if write else 0, _stream())
+
+
+ATTN_BIASED_TILE_MAX_KEY_HEAD = 128  #: the largest key head of the tile kernel (attention_biased.hip)
+
+
+def _attn_biased_common(q, out, k_cache, v_cache, gate, positions, seq_of_token, block_table, bias, far,
+                        nq, nkv, dk, dv, page_size):
+    _dev(q, out, k_cache, v_cache, gate, positions, seq_of_token, block_table, bias)
+    if not (q.dtype == out.dtype == k_cache.dtype == v_cache.dtype):
+        raise KernelError("attn_biased: queries, caches and output share one element type")
+    if tuple(k_cache.shape[1:]) != (nkv, page_size, dk) or tuple(v_cache.shape[1:]) != (nkv, page_size, dv):
+        raise KernelError("attn_biased: cache shapes do not fit the head geometry")
+    _contig("q", q), _contig("k_cache", k_cache), _contig("v_cache", v_cache)
+    if out.dim() != 2 or out.stride(1) != 1 or out.shape[1] < nq * dv:
+        raise KernelError("attn_biased: out is [N, >= nq*dv] with contiguous rows")
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise KernelError("attn_biased: block table must be int32 [rows, pages]")
+    _i32("positions", positions), _i32("seq_of_token", seq_of_token)
+    if gate is not None and (gate.dtype != torch.float32 or not gate.is_contiguous()):
+        raise KernelError("attn_biased: gates are contiguous float32 [N, nq]")
+    if bias is not None and (bias.dtype != torch.float32 or not bias.is_contiguous() or tuple(bias.shape) != (nq, far + 1)):
+        raise KernelError(f"attn_biased: the bias by distance is float32 [{nq}, {far + 1}]")
+
+
+def attn_biased_tile(q, out, k_cache, v_cache, gate, out_scale, tiles, n_tiles, positions, seq_of_token,
+                     block_table, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first) -> None:
+    """Prompt portions of the capped, biased attention; ``tiles`` is int32 [n_tiles, 2] = (first token, count <= 32)."""
+    _attn_biased_common(q, out, k_cache, v_cache, gate, positions, seq_of_token, block_table, bias, far,
+                        nq, nkv, dk, dv, page_size)
+    _i32("tiles", tiles, 2 * n_tiles)
+    call("pyre_attn_biased_tile", q.data_ptr(), out.data_ptr(), out.stride(0), dtype_code(q), k_cache.data_ptr(),
+         v_cache.data_ptr(), _ptr(gate), float(out_scale), tiles.data_ptr(), n_tiles, positions.data_ptr(),
+         seq_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0), nq, nkv, dk, dv, page_size,
+         float(scale), float(cap), _ptr(bias), int(far), int(window), int(keep_first), _stream())
+
+
+def attn_biased_single(q, out, k_cache, v_cache, gate, out_scale, tokens, n, positions, seq_of_token,
+                       block_table, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first) -> None:
+    """The same for ``n`` tokens one by one (``tokens``: which of the flat batch, None: the first n)."""
+    _attn_biased_common(q, out, k_cache, v_cache, gate, positions, seq_of_token, block_table, bias, far,
+                        nq, nkv, dk, dv, page_size)
+    if tokens is not None:
+        _dev(tokens), _i32("tokens", tokens, n)
+    call("pyre_attn_biased_single", q.data_ptr(), out.data_ptr(), out.stride(0), dtype_code(q), k_cache.data_ptr(),
+         v_cache.data_ptr(), _ptr(gate), float(out_scale), _ptr(tokens), n, positions.data_ptr(),
+         seq_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0), nq, nkv, dk, dv, page_size,
+         float(scale), float(cap), _ptr(bias), int(far), int(window), int(keep_first), _stream())
+
+
+GLA_MAX_RANK = 512     #: the widest low-rank input of the decay (linear_attention.hip)
+GLA_MAX_KEY_HEAD = 256
+GLA_MAX_VALUE_HEAD = 256
+
+
+def gla_row_width(heads: int, dk: int, dv: int) -> int:
+    """Columns of the float32 rows [q | k | log decay | v | g] that the recurrent kernels share."""
+    return 3 * heads * dk + 2 * heads * dv
+
+
+def gla_prepare(proj: Partials, col0: int, a2: torch.Tensor, a2_bias: torch.Tensor | None, tau: float,
+                x: torch.Tensor, n: int, heads: int, dk: int, dv: int) -> None:
+    """Finish the input product from column ``col0`` on (q, k: heads*dk each; v, g: heads*dv each; then the
+    low-rank input of the decay) into float32 rows ``x`` and put log(sigmoid(a2 @ low + bias)) / tau there."""
+    _dev(proj.data, a2, a2_bias, x)
+    rank = a2.shape[1]
+    args = _proj_args(proj, col0, 2 * heads * dk + 2 * heads * dv + rank)
+    if tuple(a2.shape) != (heads * dk, rank) or (a2_bias is not None and a2_bias.numel() != heads * dk):
+        raise KernelError("gla_prepare: the decay's second matrix is [heads*dk, rank], its bias [heads*dk]")
+    _contig("a2", a2)
+    if x.dtype != torch.float32 or not x.is_contiguous() or x.shape[-1] != gla_row_width(heads, dk, dv) or x.shape[0] < n \
+            or proj.rows < n:
+        raise KernelError("gla_prepare: x is contiguous float32 [>= n, 3*heads*dk + 2*heads*dv]")
+    call("pyre_gla_prepare", *args, a2.data_ptr(), dtype_code(a2), _ptr(a2_bias),
+         dtype_code(a2_bias) if a2_bias is not None else 0, float(tau), x.data_ptr(), n, heads, dk, dv, rank, _stream())
+
+
+def gla_scan(x: torch.Tensor, state: torch.Tensor, o: torch.Tensor, q_start: torch.Tensor, state_slots: torch.Tensor,
+             n_seqs: int, heads: int, dk: int, dv: int, qscale: float) -> None:
+    """The recurrence over each request's tokens of the step, from and into ``state [slots, heads, dk, dv]``;
+    ``o`` (float32 [N, heads*dv]) receives qscale * S^T q."""
+    _dev(x, state, o, q_start, state_slots)
+    for name, t in (("x", x), ("state", state), ("o", o)):
+        if t.dtype != torch.float32 or not t.is_contiguous():
+            raise KernelError(f"gla_scan: {name} is contiguous float32")
+    if tuple(state.shape[1:]) != (heads, dk, dv) or x.shape[-1] != gla_row_width(heads, dk, dv) or o.shape[-1] != heads * dv:
+        raise KernelError("gla_scan: shapes do not fit the head geometry")
+    _i32("q_start", q_start, n_seqs + 1), _i32("state_slots", state_slots, n_seqs)
+    call("pyre_gla_scan", x.data_ptr(), state.data_ptr(), o.data_ptr(), q_start.data_ptr(), state_slots.data_ptr(),
+         n_seqs, heads, dk, dv, float(qscale), _stream())
+
+
+def gla_finish(o: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: float, out_scale: float, out: torch.Tensor,
+               n: int, heads: int, dk: int, dv: int) -> None:
+    """out[n, h*dv + e] = o / rms(o over dv) * gain[e] * silu(g) * out_scale; ``out`` has contiguous rows."""
+    _dev(o, x, gain, out)
+    if o.dtype != torch.float32 or x.dtype != torch.float32 or not o.is_contiguous() or not x.is_contiguous():
+        raise KernelError("gla_finish: o and x are contiguous float32")
+    if gain.numel() != dv or out.dim() != 2 or out.stride(1) != 1 or out.shape[1] < heads * dv or out.shape[0] < n:
+        raise KernelError("gla_finish: gain [dv] and out [>= n, >= heads*dv] expected")
+    _contig("gain", gain)
+    call("pyre_gla_finish", o.data_ptr(), x.data_ptr(), gain.data_ptr(), dtype_code(gain), float(eps), float(out_scale),
+         out.data_ptr(), dtype_code(out), out.stride(0), n, heads, dk, dv, _stream())
 
 
 def rope_kv_write(qkv: Partials, q_out: torch.Tensor, k_cache: torch.Tensor | None,

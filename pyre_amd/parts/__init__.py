@@ -1,9 +1,11 @@
-from pyre_amd.parts.base import (AttentionSpec, BlockSpec, EmbeddingSpec, FeedForward,
+from pyre_amd.parts.base import (AttentionSpec, BlockSpec, CappedAttentionSpec, ClippedGLUSpec, GatedLinearAttentionSpec,
+                                 LayerNormSpec, ParallelMixerSpec, SandwichBlockSpec, EmbeddingSpec, FeedForward,
                                  LayerCall, LMHeadSpec, Mixer, ModelSpec, Norm, NoPositionSpec, Part,
                                  PagedCacheSpec, PagedTensorSpec, PositionEncoding, RMSNormSpec, RotarySpec, StateCacheSpec, SwiGLUSpec,
                                  TensorSpec, make_part, register_part)
 
-__all__ = ["AttentionSpec", "BlockSpec", "EmbeddingSpec", "FeedForward", "LayerCall",
+__all__ = ["AttentionSpec", "BlockSpec", "CappedAttentionSpec", "ClippedGLUSpec", "GatedLinearAttentionSpec",
+           "LayerNormSpec", "ParallelMixerSpec", "SandwichBlockSpec", "EmbeddingSpec", "FeedForward", "LayerCall",
            "LMHeadSpec", "Mixer", "ModelSpec", "Norm", "NoPositionSpec", "PagedCacheSpec", "PagedTensorSpec", "Part", "PositionEncoding",
            "RMSNormSpec", "RotarySpec", "StateCacheSpec", "SwiGLUSpec", "TensorSpec", "make_part",
            "register_part"]

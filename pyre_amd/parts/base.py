@@ -47,13 +47,21 @@ class TensorSpec:
     embeddings, biases: N(0, std)), ``"gain"`` (norm gains: 1 + N(0, gain_std)),
     ``"zeros"``, ``"int"`` (integer tables: zeros).
     ``alias_of`` names a tensor that stands in when this one is absent from the
-    file (a tied output head).
+    file (a tied output head). ``init`` may also be ``"normal:<std>"`` for a matrix drawn
+    with a deviation of its own.
     """
 
     name: str
-    shape: tuple[int, ...]
+    shape: tuple[int | None, ...]
     init: str = "normal"
     alias_of: str | None = None
+    #: a size that only the file knows is None in ``shape`` (the part reads it off the tensor when it
+    #: binds); the random-weights mode then draws this shape
+    random_shape: tuple[int, ...] | None = None
+
+    def fits(self, shape) -> bool:
+        shape = tuple(shape)
+        return len(shape) == len(self.shape) and all(w is None or w == g for w, g in zip(self.shape, shape))
 
 
 # --------------------------------------------------------------------------- cache needs
@@ -105,6 +113,9 @@ class PagedCacheSpec:
 
     tensors: tuple[PagedTensorSpec, ...]
     window: int = 0
+    #: with a window: the sequence's first ``keep_first`` tokens stay visible to every later query,
+    #: so the pages that hold them are never given back
+    keep_first: int = 0
     #: tokens per page that this mixer's kernels need, if they need a particular number; None:
     #: whatever the engine is set to. All page groups of an engine share one page size, so an
     #: engine set to another size refuses the model when it is built.
@@ -116,8 +127,8 @@ class PagedCacheSpec:
         names = [t.name for t in self.tensors]
         if not names or len(names) != len(set(names)):
             raise ValueError("a paged cache needs at least one tensor, each with a name of its own")
-        if self.window < 0:
-            raise ValueError("window must not be negative")
+        if self.window < 0 or self.keep_first < 0:
+            raise ValueError("window and keep_first must not be negative")
         if self.page_size is not None and self.page_size <= 0:
             raise ValueError("page_size must be positive")
 
@@ -305,6 +316,101 @@ class AttentionSpec:
 
 
 @dataclass(frozen=True)
+class LayerNormSpec:
+    """(x - mean) / sqrt(var + eps) * gain, no bias; ``name`` is the gain's tensor."""
+
+    hidden_size: int
+    eps: float
+    name: str
+    kind: ClassVar[str] = "layernorm"
+
+
+@dataclass(frozen=True)
+class CappedAttentionSpec:
+    """Softmax attention without rotation: unit-norm queries and keys (``unit_norm``), scores times
+    ``scale``, squashed by ``softcap * tanh(s / softcap)`` (0: not), plus a learned bias by distance
+    (``bias_rows`` rows of a table per head, one per distance below half of them, the rest spaced
+    evenly in log(distance) up to ``bias_far``; None: the file says how many, 0: no bias), a window
+    of ``window`` tokens (0: all) beside the sequence's first ``keep_first``, key heads of
+    ``key_dim`` and value heads of ``value_dim`` elements, one sigmoid gate per head (``gated``).
+    Tensors: ``prefix + .q / .k / .v / .g / .o / .rel``."""
+
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    key_dim: int
+    value_dim: int
+    scale: float
+    prefix: str
+    softcap: float = 0.0
+    bias_far: float = 0.0
+    bias_rows: int | None = None
+    window: int = 0
+    keep_first: int = 0
+    unit_norm: bool = True
+    norm_eps: float = 1e-6
+    gated: bool = True
+    kind: ClassVar[str] = "capped_attention"
+
+
+@dataclass(frozen=True)
+class GatedLinearAttentionSpec:
+    """Per head a float32 state S [key_dim, value_dim]: S <- diag(a) S + k v^T, o = S^T q key_dim^-1/2,
+    a = sigmoid(A2 (A1 h) + b)^(1 / tau) per key channel (``rank``: columns of A2; None: the file says).
+    The heads' outputs are divided by their root mean square, times a gain over value_dim, times silu(G h).
+    Tensors: ``prefix + .q / .k / .v / .g / .o / .norm / .a1 / .a2 / .a2.b``."""
+
+    hidden_size: int
+    num_heads: int
+    key_dim: int
+    value_dim: int
+    tau: float
+    prefix: str
+    norm_eps: float = 1e-6
+    rank: int | None = None
+    kind: ClassVar[str] = "gated_linear_attention"
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """sum_i scales[i] * branches[i](h): mixers side by side that read the same rows."""
+
+    hidden_size: int
+    branches: tuple
+    scales: tuple
+    kind: ClassVar[str] = "parallel"
+
+
+@dataclass(frozen=True)
+class ClippedGLUSpec:
+    """down(g sigmoid(slope g) (u + 1)), g = min(gate(x), limit), u = clamp(up(x), -limit, limit).
+    Tensors: ``prefix + .gate / .up / .down``."""
+
+    hidden_size: int
+    intermediate_size: int
+    limit: float
+    prefix: str
+    slope: float = 1.702
+    kind: ClassVar[str] = "clipped_glu"
+
+
+@dataclass(frozen=True)
+class SandwichBlockSpec:
+    """x += mixer_scale * mixer_post_norm(mixer(mixer_norm(x))), then the same around the
+    feed-forward (None: the layer has none). The scales are tensors over the hidden size."""
+
+    mixer: Any
+    mixer_norm: Any
+    mixer_post_norm: Any
+    mixer_scale: str | None
+    feed_forward: Any = None
+    feed_forward_norm: Any = None
+    feed_forward_post_norm: Any = None
+    feed_forward_scale: str | None = None
+    kind: ClassVar[str] = "sandwich"
+
+
+@dataclass(frozen=True)
 class SwiGLUSpec:
     hidden_size: int
     intermediate_size: int
@@ -337,6 +443,7 @@ class LMHeadSpec:
     hidden_size: int
     name: str = "lm_head.weight"
     tied_to: str | None = None       #: embedding tensor used when the head is tied
+    scale: float = 1.0               #: the logits are multiplied by this
     kind: ClassVar[str] = "lm_head"
 
 

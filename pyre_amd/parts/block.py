@@ -6,8 +6,8 @@ from dataclasses import dataclass
 
 import torch
 
-from pyre_amd.hip.ops import Partials
-from pyre_amd.parts.base import Block, BlockSpec, TensorSpec, make_part
+from pyre_amd.hip.ops import Partials, PostNorm
+from pyre_amd.parts.base import Block, BlockSpec, SandwichBlockSpec, TensorSpec, make_part, take
 
 
 @dataclass
@@ -55,3 +55,70 @@ class PreNormBlock(Block):
         mixed = self.mixer.forward(ctx, h, caches[0] if caches else None)
         self.feed_forward_norm.forward(ctx, state.resid, mixed, h)
         state.pending = self.feed_forward.forward(ctx, h)
+
+
+class SandwichBlock(Block):
+    """x += s1 * post1(mixer(norm1(x))); x += s2 * post2(feed_forward(norm2(x))): every sublayer is
+    normed before and after, and its normed result is scaled element by element before it is added.
+    The post-norms never run as kernels of their own: a sublayer's result is handed on as the pending
+    term together with its norm and scale, and the next norm's kernel applies them as it adds. A layer
+    without a feed-forward is the first half alone. A mixer made of several (``cache_specs`` on the
+    mixer) gets all of the block's cache views, a plain one its own."""
+
+    def __init__(self, spec: SandwichBlockSpec):
+        self.spec = spec
+        self.mixer = make_part("mixer", spec.mixer)
+        self.mixer_norm = make_part("norm", spec.mixer_norm)
+        self.mixer_post = make_part("norm", spec.mixer_post_norm)
+        self.feed_forward = self.feed_forward_norm = self.feed_forward_post = None
+        if spec.feed_forward is not None:
+            self.feed_forward = make_part("feed_forward", spec.feed_forward)
+            self.feed_forward_norm = make_part("norm", spec.feed_forward_norm)
+            self.feed_forward_post = make_part("norm", spec.feed_forward_post_norm)
+        self.scales: dict[str, torch.Tensor] = {}
+
+    def parts(self):
+        return tuple(p for p in (self.mixer_norm, self.mixer, self.mixer_post, self.feed_forward_norm,
+                                 self.feed_forward, self.feed_forward_post) if p is not None)
+
+    def _scale_names(self):
+        return [n for n in (self.spec.mixer_scale, self.spec.feed_forward_scale if self.feed_forward else None) if n]
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        hidden = self.mixer_norm.spec.hidden_size
+        return [s for p in self.parts() for s in p.tensor_specs()] + \
+               [TensorSpec(n, (hidden,), init="gain") for n in self._scale_names()]
+
+    def bind(self, tensors, runtime) -> None:
+        for p in self.parts():
+            p.bind(tensors, runtime)
+        for n in self._scale_names():
+            self.scales[n] = take(tensors, n).contiguous()
+
+    def linears(self) -> list:
+        return [lin for p in self.parts() for lin in p.linears()]
+
+    def cache_specs(self) -> list:
+        if hasattr(self.mixer, "cache_specs"):
+            return list(self.mixer.cache_specs())
+        spec = self.mixer.cache_spec()
+        return [] if spec is None else [spec]
+
+    def step_arrays(self) -> list:
+        return self.mixer.step_arrays()
+
+    def _post(self, term: Partials, norm, scale_name) -> Partials:
+        if term.post is not None:
+            raise ValueError("a sublayer's result already carries a norm")
+        return Partials(term.data, term.bias, PostNorm(norm.gain, norm.spec.eps, self.scales.get(scale_name)))
+
+    def forward(self, ctx, state: Hidden, caches: list) -> None:
+        h = ctx.workspace.get("block.h", (ctx.n_tokens, state.resid.shape[1]), ctx.dtype)
+        self.mixer_norm.forward(ctx, state.resid, state.pending, h)
+        cache = caches if hasattr(self.mixer, "cache_specs") else (caches[0] if caches else None)
+        state.pending = self._post(self.mixer.forward(ctx, h, cache), self.mixer_post, self.spec.mixer_scale)
+        if self.feed_forward is None:
+            return
+        self.feed_forward_norm.forward(ctx, state.resid, state.pending, h)
+        state.pending = self._post(self.feed_forward.forward(ctx, h), self.feed_forward_post,
+                                   self.spec.feed_forward_scale)

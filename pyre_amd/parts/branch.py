@@ -1,0 +1,130 @@
+"""Mixers whose matrix products can be shared: several of them side by side read the same rows,
+so their input products are one product over the row-wise concatenation of their matrices, and
+their scaled results are one output product over the column-wise concatenation of theirs."""
+
+from __future__ import annotations
+
+import torch
+
+from pyre_amd.hip.ops import Partials
+from pyre_amd.parts.base import Mixer, ParallelMixerSpec, TensorSpec, make_part, take
+from pyre_amd.parts.linear import Linear
+
+
+class BranchMixer(Mixer):
+    """A mixer of the form out(f(in_1 h, in_2 h, ...)): all its input matrices multiply the rows it is
+    given, and one output matrix multiplies what it makes of them. It says which matrices these are
+    and does the part in between (``attend``); the products are run here when it stands alone, or by a
+    :class:`ParallelMixer` for all its branches at once.
+
+    A subclass provides ``hidden_size``, ``inner`` (columns of the rows that ``attend`` writes),
+    ``in_tensors()`` (the input matrices in the order of the product's columns), ``out_tensor()``,
+    ``other_tensors()`` / ``bind_others()`` for what else it owns, and
+    ``attend(ctx, proj, col0, cache, o, scale)``: from the input product's partial sums (its own
+    columns start at ``col0``) to ``o [n, inner]`` (rows ``o.stride(0)`` apart), times ``scale``."""
+
+    hidden_size: int
+    inner: int
+    role = "mix"
+
+    def in_tensors(self) -> list[TensorSpec]:
+        raise NotImplementedError
+
+    def out_tensor(self) -> TensorSpec:
+        raise NotImplementedError
+
+    def other_tensors(self) -> list[TensorSpec]:
+        return []
+
+    def bind_others(self, tensors, runtime) -> None:
+        pass
+
+    def attend(self, ctx, proj: Partials, col0: int, cache, o: torch.Tensor, scale: float) -> None:
+        raise NotImplementedError
+
+    # ---- standing alone
+    def tensor_specs(self) -> list[TensorSpec]:
+        return [*self.in_tensors(), self.out_tensor(), *self.other_tensors()]
+
+    def bind(self, tensors, runtime) -> None:
+        w = _stacked([s.name for s in self.in_tensors()], tensors, 0)  # a size that only the file knows is known now
+        self._in = Linear(self.hidden_size, w.shape[0], f"{self.role}.in")
+        self._out = Linear(self.inner, self.hidden_size, f"{self.role}.out")
+        self._in.set(w)
+        self._out.set(take(tensors, self.out_tensor().name))
+        self.bind_others(tensors, runtime)
+
+    def linears(self) -> list:
+        return [self._in, self._out]
+
+    def forward(self, ctx, h, cache):
+        n = ctx.n_tokens
+        proj = self._in.forward(ctx, h, n)
+        o = ctx.workspace.get(f"{self.role}.o", (n, self.inner), ctx.dtype)
+        self.attend(ctx, proj, 0, cache, o, 1.0)
+        return self._out.forward(ctx, o, n)
+
+
+def _stacked(names, tensors, dim):
+    """The named tensors concatenated along ``dim``, each let go of as soon as it is copied."""
+    parts = [take(tensors, n) for n in names]
+    if len(parts) == 1:
+        return parts[0]
+    fused = torch.cat(parts, dim=dim)
+    del parts
+    return fused
+
+
+class ParallelMixer(Mixer):
+    """sum_i scale_i * branch_i(h). One input product for all branches, one output product over
+    [scale_0 o_0 | scale_1 o_1 | ...] against [Wo_0 | Wo_1 | ...]; every branch keeps its own cache
+    (``cache_specs``: one description per branch that keeps something, in their order)."""
+
+    def __init__(self, spec: ParallelMixerSpec):
+        if len(spec.branches) != len(spec.scales) or not spec.branches:
+            raise ValueError("parallel mixer: one scale per branch, at least one branch")
+        self.spec = spec
+        self.branches = [make_part("mixer", b) for b in spec.branches]
+        for b in self.branches:
+            if not isinstance(b, BranchMixer):
+                raise ValueError(f"parallel mixer: {type(b).__name__} cannot share its products")
+        self.inner = sum(b.inner for b in self.branches)
+        self.proj = self.out = None   # made when the tensors are bound: a size may be the file's to say
+        self.first_column: list[int] = []
+
+    def cache_specs(self) -> list:
+        return [s for s in (b.cache_spec() for b in self.branches) if s is not None]
+
+    def step_arrays(self) -> list:
+        return [a for b in self.branches for a in b.step_arrays()]
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return [s for b in self.branches for s in (*b.in_tensors(), b.out_tensor(), *b.other_tensors())]
+
+    def bind(self, tensors, runtime) -> None:
+        col = 0
+        self.first_column = []
+        for b in self.branches:
+            self.first_column.append(col)
+            col += sum(tensors[s.name].shape[0] for s in b.in_tensors())
+        self.proj = Linear(self.spec.hidden_size, col, "mix.in")
+        self.out = Linear(self.inner, self.spec.hidden_size, "mix.out")
+        self.proj.set(_stacked([s.name for b in self.branches for s in b.in_tensors()], tensors, 0))
+        self.out.set(_stacked([b.out_tensor().name for b in self.branches], tensors, 1))
+        for b in self.branches:
+            b.bind_others(tensors, runtime)
+
+    def linears(self) -> list:
+        return [self.proj, self.out]
+
+    def forward(self, ctx, h, caches):
+        n = ctx.n_tokens
+        proj = self.proj.forward(ctx, h, n)
+        o = ctx.workspace.get("mix.o", (n, self.inner), ctx.dtype)
+        views = iter(caches or [])
+        at = 0
+        for b, scale, col in zip(self.branches, self.spec.scales, self.first_column):
+            cache = next(views) if b.cache_spec() is not None else None
+            b.attend(ctx, proj, col, cache, o[:, at:at + b.inner], float(scale))
+            at += b.inner
+        return self.out.forward(ctx, o, n)

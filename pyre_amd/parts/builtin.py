@@ -2,10 +2,13 @@
 
 from pyre_amd.parts.attention import Attention
 from pyre_amd.parts.base import register_part
-from pyre_amd.parts.block import PreNormBlock
+from pyre_amd.parts.block import PreNormBlock, SandwichBlock
+from pyre_amd.parts.branch import ParallelMixer
+from pyre_amd.parts.capped_attention import CappedAttention
 from pyre_amd.parts.embedding import LMHead, TokenEmbedding
-from pyre_amd.parts.feedforward import SwiGLU
-from pyre_amd.parts.norm import RMSNorm
+from pyre_amd.parts.feedforward import ClippedGLU, SwiGLU
+from pyre_amd.parts.linear_attention import GatedLinearAttention
+from pyre_amd.parts.norm import LayerNorm, RMSNorm
 from pyre_amd.parts.rotary import NoPosition, RotaryEncoding
 
 register_part("mixer", "attention", Attention)
@@ -16,3 +19,9 @@ register_part("position", "none", NoPosition)
 register_part("block", "pre_norm", PreNormBlock)
 register_part("embedding", "embedding", TokenEmbedding)
 register_part("head", "lm_head", LMHead)
+register_part("mixer", "capped_attention", CappedAttention)
+register_part("mixer", "gated_linear_attention", GatedLinearAttention)
+register_part("mixer", "parallel", ParallelMixer)
+register_part("feed_forward", "clipped_glu", ClippedGLU)
+register_part("norm", "layernorm", LayerNorm)
+register_part("block", "sandwich", SandwichBlock)

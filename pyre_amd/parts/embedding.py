@@ -48,4 +48,6 @@ class LMHead(Part):
         p = self.linear.forward(ctx, h, m, out=out)
         if p.data.data_ptr() != out.data_ptr() or p.count != 1 or p.bias is not None:
             ops.reduce_partials(p, out, m)
+        if self.spec.scale != 1.0:
+            ops.scale_(out, self.spec.scale)
         return out

@@ -6,7 +6,7 @@ import torch
 
 from pyre_amd.hip import ops
 from pyre_amd.parts import fast
-from pyre_amd.parts.base import FeedForward, SwiGLUSpec, TensorSpec, take
+from pyre_amd.parts.base import ClippedGLUSpec, FeedForward, SwiGLUSpec, TensorSpec, take
 from pyre_amd.parts.linear import Linear, linear_specs
 
 
@@ -41,4 +41,39 @@ class SwiGLU(FeedForward):
         if not fast.gate_up_silu(self.gate_up, ctx, h, n, act):
             gu = self.gate_up.forward(ctx, h, n)
             ops.silu_mul(gu, act, n)
+        return self.down.forward(ctx, act, n)
+
+
+class ClippedGLU(FeedForward):
+    """down(g * sigmoid(slope * g) * (u + 1)) with g = min(gate(x), limit), u = clamp(up(x), -limit, limit):
+    a gated unit whose inputs are clipped and whose linear half is shifted by one. gate and up are one
+    product over [Wgate; Wup]."""
+
+    def __init__(self, spec: ClippedGLUSpec):
+        self.spec = spec
+        self.gate_up = Linear(spec.hidden_size, 2 * spec.intermediate_size, "ffn.gate_up")
+        self.down = Linear(spec.intermediate_size, spec.hidden_size, "ffn.down")
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        s, p = self.spec, self.spec.prefix
+        return [TensorSpec(f"{p}.gate", (s.intermediate_size, s.hidden_size)),
+                TensorSpec(f"{p}.up", (s.intermediate_size, s.hidden_size)),
+                TensorSpec(f"{p}.down", (s.hidden_size, s.intermediate_size))]
+
+    def bind(self, tensors, runtime) -> None:
+        p = self.spec.prefix
+        halves = [take(tensors, f"{p}.gate"), take(tensors, f"{p}.up")]
+        fused = torch.cat(halves, dim=0)
+        del halves
+        self.gate_up.set(fused)
+        self.down.set(take(tensors, f"{p}.down"))
+
+    def linears(self) -> list:
+        return [self.gate_up, self.down]
+
+    def forward(self, ctx, h):
+        n = ctx.n_tokens
+        act = ctx.workspace.get("ffn.act", (n, self.spec.intermediate_size), ctx.dtype)
+        gu = self.gate_up.forward(ctx, h, n)
+        ops.clipped_glu(gu, act, n, self.spec.limit, self.spec.slope)
         return self.down.forward(ctx, act, n)

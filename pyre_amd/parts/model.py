@@ -109,8 +109,15 @@ class LayeredModel(Part):
         rows = state.resid[:ctx.n_tokens].clone()
         p = state.pending
         if p is not None:
+            term = torch.zeros_like(rows)
             for i in range(p.count):
-                rows += p.data[i, :ctx.n_tokens].float()
+                term += p.data[i, :ctx.n_tokens].float()
             if p.bias is not None:
-                rows += p.bias.float()
+                term += p.bias.float()
+            if p.post is not None:  # the term's own norm and scale, as the next norm's kernel applies them
+                dev = term - term.mean(-1, keepdim=True)
+                term = dev / torch.sqrt((dev * dev).mean(-1, keepdim=True) + p.post.eps) * p.post.gain.float()
+                if p.post.scale is not None:
+                    term = term * p.post.scale.float()
+            rows += term
         return rows

@@ -1,6 +1,6 @@
 """One registry from an architecture's name to its configuration class and model builder.
 
-``config.json`` names the architecture in ``architectures[0]``; everything in the
+``config.json`` names the architecture in ``architectures[0]`` (or in ``architecture``, one string); everything in the
 framework (loader, engine, replay tool, command line) finds the model through
 this table and nowhere else. The reference accepts any name containing "Qwen2"
 (`pyre/config.py:38-43`); here the key must match exactly.
@@ -53,8 +53,10 @@ def get_architecture(name: str) -> Architecture:
 
 def architecture_of(raw: dict[str, Any]) -> Architecture:
     archs = raw.get("architectures")
+    if isinstance(raw.get("architecture"), str) and not archs:
+        archs = [raw["architecture"]]  # a design that names itself with one string
     if not archs or not isinstance(archs, (list, tuple)):
-        raise ConfigError("config.json has no 'architectures' list")
+        raise ConfigError("config.json has neither an 'architectures' list nor an 'architecture' name")
     return get_architecture(archs[0])
 
 

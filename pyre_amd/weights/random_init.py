@@ -37,8 +37,13 @@ def random_state(specs: list[TensorSpec], seed: int, std: float = 0.02, gain_std
     for s in specs:
         if s.alias_of is not None:
             continue
-        if s.init == "normal":
-            t = torch.randn(s.shape, generator=gen, dtype=torch.float32, device=device) * std
+        shape = s.random_shape if s.random_shape is not None else s.shape
+        if any(d is None for d in shape):
+            raise ValueError(f"tensor {s.name}: a size that only a file knows ({s.shape}) and no shape to draw")
+        s = TensorSpec(s.name, tuple(shape), s.init)
+        if s.init.startswith("normal"):
+            own = float(s.init.split(":", 1)[1]) if ":" in s.init else std
+            t = torch.randn(s.shape, generator=gen, dtype=torch.float32, device=device) * own
         elif s.init == "gain":
             t = torch.ones(s.shape, dtype=torch.float32, device=device)
             if gain_std:
