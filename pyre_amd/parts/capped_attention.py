@@ -78,7 +78,8 @@ class CappedAttention(BranchMixer):
         s = self.spec
         if s.bias_rows == 0:
             return []
-        return [TensorSpec(f"{s.prefix}.rel", (s.bias_rows, s.num_heads),
+        # random weights: drawn wide, so that the bias of a distance matters beside the scores
+        return [TensorSpec(f"{s.prefix}.rel", (s.bias_rows, s.num_heads), init="normal:1.0",
                            random_shape=(s.bias_rows or DEFAULT_BIAS_ROWS, s.num_heads))]
 
     def bind_others(self, tensors, runtime) -> None:

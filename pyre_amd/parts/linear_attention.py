@@ -49,7 +49,8 @@ class GatedLinearAttention(BranchMixer):
         s, p = self.spec, self.spec.prefix
         hk = s.num_heads * s.key_dim
         return [TensorSpec(f"{p}.a2", (hk, s.rank), random_shape=(hk, self._rank())),
-                TensorSpec(f"{p}.a2.b", (hk,)), TensorSpec(f"{p}.norm", (s.value_dim,), init="gain")]
+                TensorSpec(f"{p}.a2.b", (hk,), init="normal:2.0"),  # random weights: slow and fast channels
+                TensorSpec(f"{p}.norm", (s.value_dim,), init="gain")]
 
     def bind_others(self, tensors, runtime) -> None:
         p = self.spec.prefix

@@ -58,8 +58,9 @@ def distance_bucket(n: int, rows: int, far: float) -> int:
 
 
 def sees(i: int, j: int, window: int, keep_first: int) -> bool:
-    """Causal, the last ``window`` positions, and the sequence's first ``keep_first`` always."""
-    return j <= i and (i - j < window or j < keep_first)
+    """Causal, the last ``window`` positions, and the sequence's first ``keep_first`` always
+    (no window, written as 0: every earlier position)."""
+    return j <= i and (not window or i - j < window or j < keep_first)
 
 
 # ----------------------------------------------------------------------------- the softmax branch
@@ -78,7 +79,8 @@ def capped_biased_attention(h, w, p, c, eps):
     rel = w[f"{p}.rel"]                                          # [rows, H]
     rows = rel.shape[0]
     cap = c.get("softcap")
-    window, keep = c["mask"]["size"], c["mask"]["keep_first"]
+    mask = c.get("mask") or {}
+    window, keep = mask.get("size") or 0, mask.get("keep_first") or 0
     i, j = torch.arange(T)[:, None], torch.arange(T)[None, :]
     seen = torch.tensor([[sees(a, b, window, keep) for b in range(T)] for a in range(T)])
     row_of = torch.tensor([distance_bucket(n, rows, c["bias_max"]) for n in range(T)])

@@ -1,0 +1,445 @@
+"""The Mafurax design through the engine against the plain implementation (``plain_mafurax``):
+whole prompts layer by layer, prefill against token-by-token decoding, portions down to two tokens,
+mixed batches with pages and slots used again, long decoding past every window, keys made to stand
+out at the edges of a window and among the kept first tokens, a state that must survive hundreds of
+tokens, each mixer alone, the norm and the activation alone, greedy generation through the
+scheduler, and the trace replay program as a process."""
+
+from __future__ import annotations
+
+import copy
+import json
+from dataclasses import dataclass
+from typing import ClassVar
+
+import numpy as np
+import pytest
+import torch
+
+import mafurax_models as M
+import plain_mafurax as P
+from helpers import cut, first_bad, random_ids, replay
+from pyre_amd.config.model import ModelConfig
+
+pytestmark = pytest.mark.gpu
+
+#: bounds on max |difference| / max |logit| of a position, fixed before the first run: float32 against
+#: the float64 plain run; bfloat16 loosely, because the sharp softmax of these models amplifies the
+#: rounding of queries and keys (the float32 runs are the exact ones)
+TOL = {"float32": 2e-5, "bfloat16": 8e-2}
+MODELS = {"small": (M.SMALL, 11), "ones": (M.ONES, 12), "wide": (M.WIDE, 13)}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    from pyre_amd.registry import config_from_dict
+    from pyre_amd.weights import write_random_model
+
+    out = {}
+    for name, (raw, seed) in MODELS.items():
+        d = tmp_path_factory.mktemp("mafurax_" + name)
+        write_random_model(d, config_from_dict(raw), seed=seed, std=0.2, gain_std=0.2)
+        out[name] = (d, *P.read_folder(d))
+    return out
+
+
+def engine_of(folder, dtype, **kw):
+    from pyre_amd.config.engine import EngineConfig
+    from pyre_amd.engine.engine import Engine
+
+    args = dict(dtype=dtype, page_size=8, max_cached_tokens=1024, max_num_seqs=4, max_num_batched_tokens=512,
+                use_graphs=False)
+    args.update(kw)
+    return Engine.from_folder(folder, EngineConfig(**args))
+
+
+def plain_rows(cfg, w, ids):
+    return P.forward(cfg, w, ids).float()
+
+
+def whole(reqs):
+    return [([(r, ids, list(range(len(ids))))], [r]) for r, ids in reqs.items()]
+
+
+def in_portions(reqs, sizes):
+    steps = []
+    for r, ids in reqs.items():
+        pos, parts = 0, cut(len(ids), sizes)
+        for k, n in enumerate(parts):
+            steps.append(([(r, ids[pos:pos + n], list(range(n)))], [r] if k == len(parts) - 1 else []))
+            pos += n
+    return steps
+
+
+def one_by_one(reqs, first):
+    steps = []
+    for r, ids in reqs.items():
+        steps.append(([(r, ids[:first], list(range(first)))], []))
+        steps += [([(r, [ids[t]], [0])], [r] if t == len(ids) - 1 else []) for t in range(first, len(ids))]
+    return steps
+
+
+def assert_close(got, want, tol):
+    bad, worst = first_bad(got, want, tol)
+    assert bad is None, bad
+    return worst
+
+
+# ----------------------------------------------------------------------------- whole prompts, layer by layer
+
+
+@pytest.mark.parametrize("name", list(MODELS))
+def test_every_layer_of_a_whole_prompt(name, folders):
+    from pyre_amd.engine.batch import Entry
+
+    folder, cfg, w = folders[name]
+    ids = random_ids(cfg["vocab"], 75, seed=3)
+    layers = []
+    want = P.forward(cfg, w, ids, layers)
+    eng = engine_of(folder, "float32")
+    seen = {}
+    got = eng.step([Entry("a", ids, list(range(len(ids))))], tap=lambda pos, rows: seen.__setitem__(pos, rows.double().cpu()))
+    for pos, ref in enumerate(layers):
+        d = float((seen[pos] - ref).abs().max() / ref.abs().max())
+        assert d <= TOL["float32"], f"layer {pos}: {d:.2e}"
+    d = float((got.double().cpu() - want).abs().max() / want.abs().max())
+    assert d <= TOL["float32"], d
+
+
+# (the model of single heads of five and three elements runs in float32 only: in 16 bits its logits are mostly rounding)
+@pytest.mark.parametrize("name,dtype,page", [("small", "float32", 8), ("small", "bfloat16", 16), ("ones", "float32", 4),
+                                             ("wide", "float32", 16), ("wide", "bfloat16", 8)])
+def test_prefill_decode_and_portions_agree_with_plain(name, dtype, page, folders):
+    folder, cfg, w = folders[name]
+    reqs = {r: random_ids(cfg["vocab"], n, seed=n) for r, n in (("a", 90), ("b", 1), ("c", 37))}
+    want = {r: plain_rows(cfg, w, ids) for r, ids in reqs.items()}
+    eng = engine_of(folder, dtype, page_size=page)
+    assert_close(replay(eng, whole(reqs)), want, TOL[dtype])
+    # most of the prompt, then token by token: the windows pass over decoded tokens
+    tail = {r: ids for r, ids in reqs.items() if len(ids) > 1}
+    assert_close(replay(eng, one_by_one(tail, 6)), want, TOL[dtype])
+    # the first tokens of a sequence one by one from the very start
+    assert_close(replay(eng, one_by_one({"c": reqs["c"][:12]}, 1)), want, TOL[dtype])
+    for sizes in ([2], [3, 2, 17, 2, 31, 5], [64, 2, 9], [7, 1, 1, 24]):
+        assert_close(replay(eng, in_portions(tail, sizes)), want, TOL[dtype])
+    eng.cache.check_invariants()
+    assert all(g.allocator.num_used == 0 for g in eng.cache.page_groups) and eng.cache.slots.num_used == 0
+
+
+@pytest.mark.parametrize("name,dtype,poison", [("small", "float32", True), ("wide", "float32", True), ("small", "bfloat16", False),
+                                               ("ones", "float32", True)])
+def test_mixed_batches_with_pages_and_slots_used_again(name, dtype, poison, folders):
+    folder, cfg, w = folders[name]
+    reqs = {r: random_ids(cfg["vocab"], n, seed=7 * n) for r, n in (("a", 61), ("b", 9), ("c", 100), ("d", 33), ("e", 2), ("f", 47))}
+    want = {r: plain_rows(cfg, w, ids) for r, ids in reqs.items()}
+    # three slots, a pool that holds three of the requests at most: everything is used again
+    eng = engine_of(folder, dtype, max_num_seqs=3, max_cached_tokens=232, debug_poison=poison)
+    fed = {r: 0 for r in reqs}
+    live, waiting, steps, k = [], list(reqs), [], 0
+    while live or waiting:
+        while waiting and len(live) < 3:
+            live.append(waiting.pop(0))
+        entries, end = [], []
+        for r in live:
+            n = min([5, 1, 13, 2, 1, 40, 1][k % 7], len(reqs[r]) - fed[r])
+            k += 1
+            entries.append((r, reqs[r][fed[r]:fed[r] + n], list(range(n))))
+            fed[r] += n
+            if fed[r] == len(reqs[r]):
+                end.append(r)
+        steps.append((entries, end))
+        live = [r for r in live if r not in end]
+    assert_close(replay(eng, steps), want, TOL[dtype])
+    eng.cache.check_invariants()
+    assert all(g.allocator.num_used == 0 for g in eng.cache.page_groups) and eng.cache.slots.num_used == 0
+
+
+def test_long_decoding_in_a_pool_that_only_windows_make_fit(folders):
+    """260 tokens one by one through a model whose layers all have windows: its pages go back as the
+    windows pass (the kept first ones stay), so a pool of 64 tokens is enough."""
+    raw = copy.deepcopy(M.SMALL)
+    raw["layers"] = [raw["layers"][0], raw["layers"][2]]
+    folder, cfg, w = _folder_of(raw, 21)
+    ids = random_ids(cfg["vocab"], 260, seed=1)
+    want = {"a": plain_rows(cfg, w, ids)}
+    eng = engine_of(folder, "float32", page_size=8, max_cached_tokens=64, max_model_len=512, debug_poison=True)
+    assert_close(replay(eng, one_by_one({"a": ids}, 2)), want, TOL["float32"])
+    assert eng.cache.page_groups[0].allocator.num_used == 0
+
+
+_made = {}
+
+
+def _folder_of(raw, seed, tensors=None):
+    """A model folder for ``raw`` (cached by its text); ``tensors(state)`` may change the drawn weights."""
+    import tempfile
+
+    from safetensors.torch import save_file
+
+    from pyre_amd.registry import config_from_dict
+    from pyre_amd.weights import model_tensor_specs, random_state
+
+    key = (json.dumps(raw, sort_keys=True), seed, tensors)
+    if key not in _made:
+        d = tempfile.mkdtemp(prefix="mafurax_")
+        cfg = config_from_dict(raw)
+        cfg.save(d)
+        state = random_state(model_tensor_specs(cfg), seed, 0.2, 0.2)
+        if tensors is not None:
+            tensors(state)
+        save_file({k: v.contiguous() for k, v in state.items()}, d + "/model.safetensors")
+        _made[key] = (d, *P.read_folder(d))
+    return _made[key]
+
+
+# ----------------------------------------------------------------------------- keys made to stand out
+
+
+EDGE = M.model(53, 32, [M.layer(M.left(2, 1, 16, 8, 0.75, 20.0, 30, 12, 2, 8), M.right(1, 8, 8, 2.0, 2), 1.0, 0.3, ff=24, limit=2.0)],
+               eps=1e-5, logit_scale=1.0)
+
+
+def _keys_like_queries(state):
+    # keys made by the first head's query matrix: a token's key points where the same token's query
+    # points, so a query gives nearly all its weight to earlier copies of its own token
+    state["l0.mix.left.k"] = state["l0.mix.left.q"][:16].clone()
+
+
+def test_a_copy_of_the_token_at_the_windows_edge_and_among_the_first():
+    folder, cfg, w = _folder_of(EDGE, 31, _keys_like_queries)
+    window, keep, T = 12, 2, 52
+    eng = engine_of(folder, "float32", page_size=8)
+    base = [1 + (i % 50) for i in range(60)]           # no token twice within 50 positions; T appears nowhere
+    cases = {"inside": (40, 40 - (window - 1)), "outside": (40, 40 - window), "first": (40, keep - 1), "after_first": (40, keep),
+             "page_border": (47, 40), "far": (57, 9)}
+    reqs = {}
+    for name, (i, j) in cases.items():
+        ids = list(base)
+        ids[i] = ids[j] = T
+        reqs[name] = ids
+    want = {r: plain_rows(cfg, w, ids) for r, ids in reqs.items()}
+    # the construction works: whether the copy is seen decides the logits at the query
+    seen = float((want["inside"][40] - want["outside"][40]).abs().max() / want["inside"][40].abs().max())
+    kept = float((want["first"][40] - want["after_first"][40]).abs().max() / want["first"][40].abs().max())
+    assert seen > 500 * TOL["float32"] and kept > 500 * TOL["float32"], (seen, kept)
+    for steps in (whole(reqs), one_by_one(reqs, 30), in_portions(reqs, [39, 2, 5]), in_portions(reqs, [2, 3])):
+        assert_close(replay(eng, steps), want, TOL["float32"])
+
+
+def test_a_state_that_has_to_last():
+    """Decays close to one: the first tokens reach the last logits through the recurrent state alone
+    (the window is 12 tokens, two first tokens are kept, the changed token is the fourth)."""
+    def slow(state):
+        state["l0.mix.right.a2.b"] = torch.full_like(state["l0.mix.right.a2.b"], 7.0)
+        state["l0.mix.right.a2"] = state["l0.mix.right.a2"] * 0.1
+    raw = copy.deepcopy(EDGE)
+    raw["layers"][0]["mixer"]["right_scale"] = 1.5
+    folder, cfg, w = _folder_of(raw, 32, slow)
+    ids = random_ids(cfg["vocab"], 300, seed=9)
+    other = list(ids)
+    other[3] = (ids[3] + 1) % cfg["vocab"]
+    want = {"a": plain_rows(cfg, w, ids), "b": plain_rows(cfg, w, other)}
+    moved = float((want["a"][-1] - want["b"][-1]).abs().max() / want["a"][-1].abs().max())
+    assert moved > 1e-3, moved
+    eng = engine_of(folder, "float32", page_size=16, max_cached_tokens=640)
+    reqs = {"a": ids, "b": other}
+    assert_close(replay(eng, whole(reqs)), want, TOL["float32"])
+    assert_close(replay(eng, in_portions(reqs, [64, 2, 31, 100, 3])), want, TOL["float32"])
+    assert_close(replay(eng, one_by_one({"a": ids}, 250)), want, TOL["float32"])
+
+
+# ----------------------------------------------------------------------------- each mechanism alone
+
+
+@dataclass(frozen=True)
+class OneMixerConfig(ModelConfig):
+    """A model of sandwich layers whose mixer is a single branch: 'left' or 'right' of the design."""
+
+    raw: dict
+    architecture: ClassVar[str] = "ToyOneMixer"
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(raw)
+
+    def to_dict(self):
+        return self.raw
+
+    def save(self, folder):
+        import pathlib
+        pathlib.Path(folder, "config.json").write_text(json.dumps(self.raw))
+
+    def __hash__(self):
+        return id(self)
+
+
+def _build_one_mixer(cfg):
+    from pyre_amd.config.mafurax import CappedAttentionConfig, GatedLinearConfig
+    from pyre_amd.parts.base import (CappedAttentionSpec, EmbeddingSpec, GatedLinearAttentionSpec, LayerCall, LayerNormSpec,
+                                     LMHeadSpec, ModelSpec, SandwichBlockSpec)
+
+    raw = cfg.raw
+    width, eps = raw["width"], raw["norm"]["eps"]
+    layers = []
+    for i, layer in enumerate(raw["layers"]):
+        p = f"l{i}.mix"
+        if layer["type"] == "left":
+            a = CappedAttentionConfig.from_dict(layer["mixer"], "left")
+            mixer = CappedAttentionSpec(width, a.heads, a.kv_heads, a.dim, a.vdim, a.scale, p, softcap=a.softcap, bias_far=a.bias_max,
+                                        bias_rows=a.bias_rows, window=a.window, keep_first=a.keep_first, norm_eps=eps)
+        else:
+            r = GatedLinearConfig.from_dict(layer["mixer"], "right")
+            mixer = GatedLinearAttentionSpec(width, r.heads, r.dim, r.vdim, r.tau, p, norm_eps=eps, rank=r.rank)
+        layers.append(SandwichBlockSpec(mixer, LayerNormSpec(width, eps, f"l{i}.norm1"), LayerNormSpec(width, eps, f"l{i}.norm1b"),
+                                        f"l{i}.ls1"))
+    return ModelSpec(width, raw["vocab"], 0, EmbeddingSpec(raw["vocab"], width, name="embed"), tuple(layers),
+                     tuple(LayerCall(i) for i in range(len(layers))), LayerNormSpec(width, eps, "final.norm"),
+                     LMHeadSpec(raw["vocab"], width, name="embed", scale=raw["logit_scale"]))
+
+
+@pytest.mark.parametrize("kind", ["left", "right"])
+def test_each_mixer_alone(kind, tmp_path):
+    from pyre_amd.registry import register_architecture, unregister_architecture
+    from pyre_amd.weights import write_random_model
+
+    mixers = {"left": [M.left(4, 2, 24, 16, 0.5, 6.0, 40, 20, 3, 10), M.left(5, 1, 7, 9, 0.8, 0.0, 12, 0, 0, 5)],
+              "right": [M.right(2, 16, 24, 4.0, 5), M.right(3, 33, 7, 1.0, 1)]}[kind]
+    raw = {"architectures": ["ToyOneMixer"], "vocab": 71, "width": 40, "norm": {"eps": 1e-5}, "logit_scale": 0.8,
+           "layers": [{"type": kind, "mixer": m, "mlp": None} for m in mixers]}
+    P.MIXERS["left"] = P.capped_biased_attention
+    P.MIXERS["right"] = P.gated_linear_attention
+    register_architecture(OneMixerConfig.architecture, OneMixerConfig, _build_one_mixer)
+    try:
+        write_random_model(tmp_path, OneMixerConfig(raw), seed=41, std=0.2, gain_std=0.2)
+        cfg, w = P.read_folder(tmp_path)
+        reqs = {r: random_ids(71, n, seed=n) for r, n in (("a", 70), ("b", 19))}
+        want = {r: plain_rows(cfg, w, ids) for r, ids in reqs.items()}
+        eng = engine_of(tmp_path, "float32")
+        kinds = [type(s).__name__ for s in eng.model.cache_specs()[0]]
+        assert kinds == (["PagedCacheSpec"] if kind == "left" else ["StateCacheSpec"])
+        assert_close(replay(eng, whole(reqs)), want, TOL["float32"])
+        assert_close(replay(eng, in_portions(reqs, [5, 2, 30])), want, TOL["float32"])
+        assert_close(replay(eng, one_by_one(reqs, 4)), want, TOL["float32"])
+    finally:
+        unregister_architecture(OneMixerConfig.architecture)
+        P.MIXERS.pop("left"), P.MIXERS.pop("right")
+
+
+@pytest.mark.parametrize("hidden,dtype", [(48, torch.float32), (700, torch.float32), (2100, torch.bfloat16)])
+def test_layer_norm_with_a_normed_pending_term(hidden, dtype):
+    from pyre_amd.hip import ops
+
+    g = torch.Generator().manual_seed(hidden)
+    n = 9
+    resid = torch.randn(n, hidden, generator=g) * 3 + 1.5
+    parts = torch.randn(3, n, hidden, generator=g)
+    gain, pgain, scale = (1 + 0.3 * torch.randn(hidden, generator=g) for _ in range(3))
+    term = P.layer_norm(parts.double().sum(0), pgain.double(), 1e-4) * scale.double()
+    want_resid = resid.double() + term
+    want_out = P.layer_norm(want_resid, gain.double(), 1e-6)
+    dev = "cuda:0"
+    r = resid.to(dev)
+    out = torch.empty(n, hidden, device=dev, dtype=dtype)
+    ops.add_layernorm(r, ops.Partials(parts.to(dev), None, ops.PostNorm(pgain.to(dev), 1e-4, scale.to(dev))), gain.to(dev), 1e-6, out)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    assert float((r.cpu().double() - want_resid).abs().max()) < 1e-5 * float(want_resid.abs().max())
+    assert float((out.cpu().double() - want_out).abs().max()) < tol * float(want_out.abs().max())
+    # some rows only, the stream untouched
+    r2 = resid.to(dev)
+    rows = torch.tensor([7, 0, 3], dtype=torch.int32, device=dev)
+    out2 = torch.empty(3, hidden, device=dev, dtype=dtype)
+    ops.add_layernorm(r2, ops.Partials(parts.to(dev)), gain.to(dev), 1e-6, out2, rows)
+    want2 = P.layer_norm(resid.double() + parts.double().sum(0), gain.double(), 1e-6)[[7, 0, 3]]
+    assert torch.equal(r2.cpu(), resid) and float((out2.cpu().double() - want2).abs().max()) < tol * float(want2.abs().max())
+    with pytest.raises(Exception):
+        ops.add_rmsnorm(r, ops.Partials(parts.to(dev), None, ops.PostNorm(pgain.to(dev), 1e-4)), gain.to(dev), 1e-6, out)
+
+
+def test_clipped_gated_unit():
+    from pyre_amd.hip import ops
+
+    g = torch.Generator().manual_seed(5)
+    n, inter, hidden = 6, 37, 20
+    gu = torch.randn(2, n, 2 * inter, generator=g) * 2
+    total = gu.double().sum(0)
+    gate, up = total[:, :inter].clamp(max=1.5), total[:, inter:].clamp(-1.5, 1.5)
+    want = gate * torch.sigmoid(1.702 * gate) * (up + 1)
+    assert bool((total[:, :inter] > 1.5).any() and (total[:, inter:] < -1.5).any())
+    out = torch.empty(n, inter, device="cuda:0")
+    ops.clipped_glu(ops.Partials(gu.to("cuda:0")), out, n, 1.5, 1.702)
+    assert float((out.cpu().double() - want).abs().max()) < 1e-5
+    # and as the plain feed-forward has it, weights included
+    w = {"f.gate": torch.randn(inter, hidden, generator=g).double(), "f.up": torch.randn(inter, hidden, generator=g).double(),
+         "f.down": torch.eye(inter).double()}
+    h = torch.randn(n, hidden, generator=g).double()
+    ops.clipped_glu(ops.Partials(torch.cat([h @ w["f.gate"].T, h @ w["f.up"].T], 1).float()[None].contiguous().to("cuda:0")), out, n, 0.7, 1.702)
+    assert float((out.cpu().double() - P.clamped_glu(h, w, "f", {"limit": 0.7})).abs().max()) < 1e-5
+
+
+# ----------------------------------------------------------------------------- the entry points
+
+
+@pytest.mark.parametrize("graphs", [False, True])
+def test_greedy_generation_through_the_scheduler(graphs, folders):
+    from pyre_amd.api import generate, load_model
+
+    folder, cfg, w = folders["small"]
+    prompts = [random_ids(cfg["vocab"], n, seed=n + 1) for n in (1, 9, 40, 23)]
+    eng, _ = load_model(str(folder), device="cuda:0", dtype="float32", page_size=8, max_cached_tokens=1024, max_num_seqs=4,
+                        max_num_batched_tokens=64, prefill_chunk=16, use_graphs=graphs)
+    got = generate(eng, prompts, max_new_tokens=30)
+    for p, g in zip(prompts, got):
+        assert len(g) == 30
+        ids = list(p)
+        for k, tok in enumerate(g):
+            row = P.forward(cfg, w, ids)[-1]
+            twin = int(row.argmax())
+            if twin != tok:
+                margin = float((row[twin] - row[tok]) / row.abs().max())
+                assert margin < TOL["float32"], f"token {k} is {tok}, plainly {twin} (margin {margin:.2e})"
+            ids.append(tok)
+    assert all(g.allocator.num_used == 0 for g in eng.cache.page_groups) and eng.cache.slots.num_used == 0
+    if graphs:
+        assert eng.graph_replays > 0
+
+
+@pytest.mark.parametrize("dtype,extra", [("float32", ("--page-size", "8", "--poison")), ("bfloat16", ())])
+def test_trace_run_as_a_process(dtype, extra, folders, tmp_path):
+    from test_trace_run_gpu import run_trace
+
+    folder, cfg, w = folders["small"]
+    vocab = cfg["vocab"]
+    reqs = {"a": random_ids(vocab, 70, 1), "b": random_ids(vocab, 40, 2), "c": random_ids(vocab, 64, 3), "d": random_ids(vocab, 3, 4),
+            "e": random_ids(vocab, 61, 5)}
+    fed = {r: 0 for r in reqs}
+    sizes = [13, 2, 30, 1, 7, 64, 3]
+    live, waiting, steps, k, wanted = [], list(reqs), [], 0, {}
+    while live or waiting:
+        while waiting and len(live) < 4:
+            live.append(waiting.pop(0))
+        entries, end = [], []
+        for r in live:
+            n = min(sizes[k % len(sizes)], len(reqs[r]) - fed[r])
+            k += 1
+            want = [] if k % 5 == 0 else list(range(0, n, 2))
+            entries.append({"id": r, "tokens": reqs[r][fed[r]:fed[r] + n], "want": want})
+            wanted.setdefault(len(steps), []).extend((r, fed[r] + x) for x in want)
+            fed[r] += n
+            if fed[r] == len(reqs[r]):
+                end.append(r)
+        steps.append({"step": len(steps), "entries": entries, "end": end})
+        live = [r for r in live if r not in end]
+    out = tmp_path / "out"
+    run_trace(folder, dtype, out, 4 * 128, steps, extra)
+    ref = {r: plain_rows(cfg, w, ids) for r, ids in reqs.items()}
+    checked = 0
+    for st, rows in wanted.items():
+        if not rows:
+            assert not (out / f"{st}.f32").exists()
+            continue
+        got = torch.from_numpy(np.fromfile(out / f"{st}.f32", dtype="<f4").reshape(len(rows), vocab))
+        for i, (r, pos) in enumerate(rows):
+            d = float((got[i] - ref[r][pos]).abs().max() / ref[r][pos].abs().max())
+            assert d <= TOL[dtype], f"step {st} request {r} position {pos}: {d:.3e}"
+            checked += 1
+    assert checked > 50
