@@ -8,6 +8,7 @@
 //              z = A2 (A1 h) + b,  ld = log(sigmoid(z)) / tau  (so that a = sigmoid(z)^(1/tau)).
 // gla_scan     walks the tokens of every request of the step in their order from the state that
 //              earlier steps left in the request's slot, and leaves the new state there.
+// gla_chunks   the same for requests that bring many tokens, sixteen tokens at a time.
 // gla_finish   divides every head's output by its root mean square, times a gain over dv that the
 //              heads share, times silu(g) and a scale; writes the rows that the output product reads.
 //
@@ -99,6 +100,109 @@ __global__ __launch_bounds__(kThreads) void gla_scan_kernel(
   }
 }
 
+// The same recurrence for requests that bring many tokens: chunks of 16 tokens, each worked on by the
+// whole block at once, so that the chain of dependent steps is a sixteenth as long. With b_t the sum
+// of the chunk's log decays up to and including token t (per key channel) and B = b of its last token:
+//
+//   o_t = qscale * ( (q_t * exp(b_t))^T S_prev + sum_{s <= t} A[t][s] v_s ),   A[t][s] = sum_d q_td k_sd exp(b_td - b_sd)
+//   S   = diag(exp(B)) S_prev + sum_s (k_s * exp(B - b_s)) v_s^T
+//
+// Every exponent is <= 0 (a decay never grows), whatever the decays are: the pair (t, s) gets its own
+// exponentials instead of a product of two factors that could overflow. Same block shape and state
+// layout as gla_scan; q, k and b of the chunk lie in LDS (dynamic: 3 * 16 * dk floats).
+constexpr int kChunk = 16;
+
+template <int DR>
+__global__ __launch_bounds__(kThreads) void gla_chunk_kernel(
+    const float* __restrict__ x, float* __restrict__ state, float* __restrict__ o, const int* __restrict__ q_start,
+    const int* __restrict__ state_slots, int heads, int dk, int dv, float qscale) {
+  extern __shared__ float chunk_lds[];
+  float* qs = chunk_lds;               // [kChunk][dk]: q, later q * exp(b)
+  float* ks = qs + kChunk * dk;        // [kChunk][dk]: k, later k * exp(B - b)
+  float* bs = ks + kChunk * dk;        // [kChunk][dk]: log decays, then their running sums
+  __shared__ float vs[kChunk][kWave];
+  __shared__ float A[kChunk][kChunk + 1];
+  __shared__ float red[4][kChunk][kWave];
+  const int s = blockIdx.x, hd = blockIdx.y, tid = threadIdx.x, w = tid >> 6, lane = tid & 63;
+  const int col = blockIdx.z * kWave + lane;
+  const bool has_col = col < dv;
+  const int t_begin = q_start[s], t_end = q_start[s + 1];
+  const int hk = heads * dk, hv = heads * dv, width = 3 * hk + 2 * hv;
+  float* st = state + (static_cast<size_t>(state_slots[s]) * heads + hd) * dk * dv;
+  float S[DR];
+#pragma unroll
+  for (int r = 0; r < DR; ++r) {
+    const int row = w + 4 * r;
+    S[r] = has_col && row < dk ? st[static_cast<size_t>(row) * dv + col] : 0.f;
+  }
+  for (int t0 = t_begin; t0 < t_end; t0 += kChunk) {
+    const int nc = min(kChunk, t_end - t0);
+    for (int i = tid; i < nc * dk; i += kThreads) {
+      const int t = i / dk, d = i % dk;
+      const float* xr = x + static_cast<size_t>(t0 + t) * width + hd * dk + d;
+      qs[i] = xr[0];
+      ks[i] = xr[hk];
+      bs[i] = xr[2 * hk];
+    }
+    for (int i = tid; i < nc * kWave; i += kThreads) {
+      const int t = i >> 6, c = blockIdx.z * kWave + (i & 63);
+      vs[t][i & 63] = c < dv ? x[static_cast<size_t>(t0 + t) * width + 3 * hk + hd * dv + c] : 0.f;
+    }
+    __syncthreads();
+    for (int d = tid; d < dk; d += kThreads)
+      for (int t = 1; t < nc; ++t) bs[t * dk + d] += bs[(t - 1) * dk + d];
+    __syncthreads();
+    // A[t][s] for s <= t: a wave a pair, its lanes over the key channels
+    for (int p = w; p < nc * (nc + 1) / 2; p += 4) {
+      int t = 0;
+      while ((t + 1) * (t + 2) / 2 <= p) ++t;
+      const int sidx = p - t * (t + 1) / 2;
+      float a = 0.f;
+      for (int d = lane; d < dk; d += kWave)
+        a = fmaf(qs[t * dk + d] * ks[sidx * dk + d], expf(bs[t * dk + d] - bs[sidx * dk + d]), a);
+      a = wave_sum(a);
+      if (lane == 0) A[t][sidx] = a;
+    }
+    __syncthreads();
+    for (int i = tid; i < nc * dk; i += kThreads) {
+      const int d = i % dk;
+      qs[i] *= expf(bs[i]);
+      ks[i] *= expf(bs[(nc - 1) * dk + d] - bs[i]);
+    }
+    __syncthreads();
+    for (int t = 0; t < nc; ++t) {
+      float part = 0.f;
+#pragma unroll
+      for (int r = 0; r < DR; ++r) {
+        const int row = w + 4 * r;
+        if (row < dk) part = fmaf(S[r], qs[t * dk + row], part);
+      }
+      red[w][t][lane] = part;
+    }
+#pragma unroll
+    for (int r = 0; r < DR; ++r) {
+      const int row = w + 4 * r;
+      if (row < dk) {
+        float add = 0.f;
+        for (int t = 0; t < nc; ++t) add = fmaf(ks[t * dk + row], vs[t][lane], add);
+        S[r] = expf(bs[(nc - 1) * dk + row]) * S[r] + add;
+      }
+    }
+    __syncthreads();
+    for (int t = w; t < nc; t += 4) {
+      float acc = ((red[0][t][lane] + red[1][t][lane]) + red[2][t][lane]) + red[3][t][lane];
+      for (int sidx = 0; sidx <= t; ++sidx) acc = fmaf(A[t][sidx], vs[sidx][lane], acc);
+      if (has_col) o[static_cast<size_t>(t0 + t) * hv + hd * dv + col] = acc * qscale;
+    }
+    __syncthreads();  // the chunk's LDS is read; the next chunk may load
+  }
+#pragma unroll
+  for (int r = 0; r < DR; ++r) {
+    const int row = w + 4 * r;
+    if (has_col && row < dk) st[static_cast<size_t>(row) * dv + col] = S[r];
+  }
+}
+
 __global__ __launch_bounds__(kThreads) void gla_finish_kernel(
     const float* __restrict__ o, const float* __restrict__ x, const void* __restrict__ gain, int gain_dt, float eps,
     float out_scale, void* __restrict__ out, int out_dt, int out_ld, int heads, int dk, int dv) {
@@ -155,6 +259,23 @@ extern "C" int pyre_gla_scan(const float* x, float* state, float* o, const int* 
   else PYRE_SCAN(64);
 #undef PYRE_SCAN
   return check_launch("gla_scan");
+}
+
+extern "C" int pyre_gla_chunks(const float* x, float* state, float* o, const int* q_start, const int* state_slots,
+                               int n_seqs, int heads, int dk, int dv, float qscale, hipStream_t stream) {
+  PYRE_REQUIRE(heads > 0 && heads <= 65535 && dk > 0 && dk <= 256 && dv > 0, "gla_chunks: heads %d, sizes %d / %d are not taken", heads, dk, dv);
+  if (n_seqs <= 0) return 0;
+  const dim3 grid(n_seqs, heads, (dv + kWave - 1) / kWave);
+  const size_t lds = sizeof(float) * 3 * kChunk * dk;
+#define PYRE_CHUNKS(DR)                                                                                              \
+  hipLaunchKernelGGL(gla_chunk_kernel<DR>, grid, dim3(kThreads), lds, stream, x, state, o, q_start, state_slots, heads, \
+                     dk, dv, qscale)
+  if (dk <= 32) PYRE_CHUNKS(8);
+  else if (dk <= 64) PYRE_CHUNKS(16);
+  else if (dk <= 128) PYRE_CHUNKS(32);
+  else PYRE_CHUNKS(64);
+#undef PYRE_CHUNKS
+  return check_launch("gla_chunks");
 }
 
 extern "C" int pyre_gla_finish(const float* o, const float* x, const void* gain, int gain_dt, float eps, float out_scale,

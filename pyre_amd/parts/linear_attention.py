@@ -64,5 +64,7 @@ class GatedLinearAttention(BranchMixer):
         x = ws.get("gla.x", (n, ops.gla_row_width(*shape)), torch.float32)
         raw = ws.get("gla.raw", (n, s.num_heads * s.value_dim), torch.float32)
         ops.gla_prepare(proj, col0, self.a2, self.a2_bias, s.tau, x, n, *shape)
-        ops.gla_scan(x, cache.tensor, raw, ctx.q_start, cache.slots, ctx.n_seqs, *shape, s.key_dim ** -0.5)
+        # single tokens walk the recurrence as it is written; prompt portions take sixteen tokens at a time
+        ops.gla_scan(x, cache.tensor, raw, ctx.q_start, cache.slots, ctx.n_seqs, *shape, s.key_dim ** -0.5,
+                     chunks=ctx.host.max_q_len > 1)
         ops.gla_finish(raw, x, self.gain, s.norm_eps, scale, o, n, *shape)
