@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--model qwen2.5-7b]
     python bench.py --workload serve [--model qwen2.5-1.5b] [--requests 256] [--max-batch 256]
+    python bench.py --workload designs [--shapes 1.5b,7b] [--layers 4]
 
 A step is one decode step of the scheduler: every running request gets one new
 token (plan, one engine step over the paged cache, greedy sampling, token fed
@@ -26,6 +27,13 @@ decode excludes prefill (`bench/harness.py:10-12`).
 scheduler run, all tokens over the wall clock): by default 256 requests on the
 Qwen2.5-1.5B shape, prompt lengths log-uniform in [16, 2048], outputs uniform in
 [16, 512], prompt portions of 512, contexts of at most 4,096, seeded.
+
+``--workload designs`` puts two designs side by side at equal width, feed-forward width, vocabulary
+and number of layers (``--layers`` of them, 4 by default, of the 1.5B and the 7B shape's layer sizes):
+the Qwen2 design and the Mafurax design, whose mixer splits the same number of heads between its
+softmax branch (window of 1,024 tokens beside 4 kept first ones) and its recurrent branch. For each:
+the prefill of a 2,048-token prompt, decode steps at 8 and 64 requests with contexts of 4,096, and
+the device time of every kernel of a prefill step and of a decode step at 8 requests.
 
 Synthetic token ids (uniform over the vocabulary), random weights ~ N(0, 0.02): there is
 no tokenizer and no checkpoint here.
@@ -186,6 +194,122 @@ def serve(args) -> dict:
     return line
 
 
+DESIGN_SHAPES = {
+    "1.5b": dict(width=1536, ff=8960, heads=12, kv_heads=2, head=128, vocab=151936),
+    "7b": dict(width=3584, ff=18944, heads=28, kv_heads=4, head=128, vocab=152064),
+}
+
+
+def designs(args) -> dict:
+    """Two designs at equal layer sizes, side by side: prefill, decode and per-kernel device times."""
+    import torch
+    from torch.profiler import ProfilerActivity, profile
+
+    from pyre_amd.api import Scheduler
+    from pyre_amd.config import EngineConfig
+    from pyre_amd.engine.context import TORCH_DTYPES
+    from pyre_amd.engine.engine import Engine
+    from pyre_amd.registry import config_from_dict
+    from pyre_amd.weights import model_tensor_specs, random_state
+
+    dev, context, layers = "cuda:0", args.context, args.layers or 4
+    rng = random.Random(0)
+
+    def configs(sh):
+        qwen = {"architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": layers, "hidden_size": sh["width"],
+                "num_attention_heads": sh["heads"], "num_key_value_heads": sh["kv_heads"], "head_dim": sh["head"],
+                "intermediate_size": sh["ff"], "vocab_size": sh["vocab"], "rope_theta": 1e6, "rms_norm_eps": 1e-6,
+                "tie_word_embeddings": True, "max_position_embeddings": 32768}
+        left = {"heads": sh["heads"] // 2, "kv_heads": max(1, sh["kv_heads"] // 2), "dim": sh["head"], "vdim": sh["head"],
+                "scale": sh["head"] ** -0.5, "softcap": 30.0, "bias_max": 1024, "bias_rows": 32,
+                "mask": {"size": 1024, "keep_first": 4}}
+        right = {"heads": sh["heads"] // 2, "dim": sh["head"], "vdim": sh["head"], "tau": 16.0, "rank": 16}
+        layer = {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0},
+                 "mlp": {"kind": "dense", "ff": sh["ff"], "limit": 7.0}}
+        mafurax = {"architecture": "Mafurax", "vocab": sh["vocab"], "width": sh["width"], "layers": [layer] * layers,
+                   "norm": {"eps": 1e-6}, "logit_scale": 1.0}
+        return {"qwen2": config_from_dict(qwen), "mafurax": config_from_dict(mafurax)}
+
+    def kernels_of(run, per: int) -> dict:
+        with profile(activities=[ProfilerActivity.CUDA]) as prof:
+            run()
+            torch.cuda.synchronize()
+        rows = sorted(((e.key, e.device_time_total, e.count) for e in prof.key_averages() if e.device_time_total > 0), key=lambda r: -r[1])
+        short = lambda k: k.replace("void ", "").replace("(anonymous namespace)::", "").replace("pyre::", "").split("(")[0][:56]  # noqa: E731
+        out = {}
+        for key, total, count in rows[:14]:
+            out[short(key)] = {"us": round(total / per, 1), "launches": round(count / per, 1)}
+        out["all kernels"] = {"us": round(sum(t for _, t, _ in rows) / per, 1)}
+        return out
+
+    def measure(name, cfg) -> dict:
+        batches = [8, 64]
+        ec = EngineConfig(dtype=args.dtype, device=dev, page_size=16, max_num_seqs=max(batches),
+                          max_cached_tokens=max(batches) * context + 1024, max_model_len=context,
+                          max_num_batched_tokens=PREFILL_TOKENS, prefill_chunk=PREFILL_TOKENS, use_graphs=not args.no_graphs)
+        state = random_state(model_tensor_specs(cfg), 0, 0.02, 0.0, TORCH_DTYPES[ec.dtype], device=dev)
+        params = sum(t.numel() for t in state.values())
+        engine = Engine.from_state(cfg, state, ec, consume=True)
+        del state
+        checked = None if args.no_gate else gate(engine, cfg.vocab_size, args.dtype, layers, name)
+        res = {"parameters": params, "gate": checked}
+
+        def prefill_once():
+            sched = Scheduler(engine, max_batch=1)
+            sched.add_request([rng.randrange(cfg.vocab_size) for _ in range(PREFILL_TOKENS)], max_new_tokens=1)
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            sched.step()
+            torch.cuda.synchronize()
+            return time.perf_counter() - t
+
+        times = [prefill_once() for _ in range(4)][1:]
+        ms = statistics.median(times) * 1e3
+        res["prefill"] = {"tokens": PREFILL_TOKENS, "ms": round(ms, 3), "tok_s": round(PREFILL_TOKENS / ms * 1e3, 1)}
+        res["prefill_kernels_us"] = kernels_of(prefill_once, 1)
+        for batch in batches:
+            sched = Scheduler(engine, max_batch=batch)
+            steps = args.steps
+            start = context - 3 * steps - args.warmup - 2 * batch - 8
+            for _ in range(batch):
+                sched.add_request([rng.randrange(cfg.vocab_size) for _ in range(start)], max_new_tokens=context - start)
+            while any(r.num_computed < len(r.prompt_ids) for r in sched.running + sched.waiting):
+                sched.step()
+            for _ in range(args.warmup):
+                sched.step()
+            blocks = []
+            for _ in range(3):
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                for _ in range(steps):
+                    sched.step()
+                torch.cuda.synchronize()
+                blocks.append(time.perf_counter() - t)
+            dt = sorted(blocks)[1]
+            res[f"decode_b{batch}"] = {"ms": round(dt / steps * 1e3, 4), "tok_s": round(batch * steps / dt, 1)}
+            if batch == batches[0]:
+                res["decode_kernels_us"] = kernels_of(lambda: [sched.step() for _ in range(4)], 4)
+            for r in list(sched.running):
+                engine.finish(r.seq_id)
+        print(f"[bench] {name}: {json.dumps({k: v for k, v in res.items() if not k.endswith('_us')})}", file=sys.stderr, flush=True)
+        del engine
+        gc.collect()
+        torch.cuda.empty_cache()
+        return res
+
+    out = {}
+    for shape in [x for x in args.shapes.split(",") if x]:
+        out[shape] = {name: measure(f"{name} {shape}", cfg) for name, cfg in configs(DESIGN_SHAPES[shape]).items()}
+    first = out[next(iter(out))]
+    return {"metric": "prefill and decode of two designs at equal layer sizes (%d layers)" % layers,
+            "value": first["mafurax"]["decode_b8"]["tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": first["mafurax"]["decode_b8"]["ms"], "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic token ids, random weights N(0, 0.02) seed 0",
+            "config": {"shapes": DESIGN_SHAPES, "layers": layers, "context": context, "prefill_tokens": PREFILL_TOKENS,
+                       "graphs": not args.no_graphs}, "designs": out, "env": environment()}
+
+
 def gate_bounds(dtype: str, layers: int) -> float:
     """How far the logits of one position may lie apart, as a part of the row's largest logit,
     when the position is computed in two ways by an engine that is in order: rounding noise of
@@ -234,7 +358,8 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--model", default=None, help="preset shape (qwen2.5-7b; for --workload serve qwen2.5-1.5b)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serve"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "designs"])
+    ap.add_argument("--shapes", default="1.5b,7b", help="designs: the layer sizes to compare at (1.5b, 7b)")
     ap.add_argument("--requests", type=int, default=256, help="serve: number of requests")
     ap.add_argument("--max-batch", type=int, default=256, help="serve: requests that run at a time")
     ap.add_argument("--seed", type=int, default=0, help="serve: seed of the lengths and token ids")
@@ -264,6 +389,9 @@ def main() -> int:
         return 2
     if args.workload == "serve":
         print(json.dumps(serve(args)))
+        return 0
+    if args.workload == "designs":
+        print(json.dumps(designs(args)))
         return 0
     plain_run = (args.model is None and args.batch == 8 and args.context == 4096 and args.points == "1,64" and args.dtype == "bfloat16"
                  and args.layers is None and not (args.no_prefill or args.prefill_only or args.no_graphs or args.opt))

@@ -8,7 +8,7 @@
 //              z = A2 (A1 h) + b,  ld = log(sigmoid(z)) / tau  (so that a = sigmoid(z)^(1/tau)).
 // gla_scan     walks the tokens of every request of the step in their order from the state that
 //              earlier steps left in the request's slot, and leaves the new state there.
-// gla_chunks   the same for requests that bring many tokens, sixteen tokens at a time.
+// gla_chunks   the same for requests that bring many tokens, sixteen tokens at a time on the matrix cores.
 // gla_finish   divides every head's output by its root mean square, times a gain over dv that the
 //              heads share, times silu(g) and a scale; writes the rows that the output product reads.
 //
@@ -100,107 +100,159 @@ __global__ __launch_bounds__(kThreads) void gla_scan_kernel(
   }
 }
 
-// The same recurrence for requests that bring many tokens: chunks of 16 tokens, each worked on by the
-// whole block at once, so that the chain of dependent steps is a sixteenth as long. With b_t the sum
-// of the chunk's log decays up to and including token t (per key channel) and B = b of its last token:
+// The same recurrence for requests that bring many tokens: chunks of 16 tokens, each worked on by a
+// whole block at once on the matrix cores' float32 instruction, so that the chain of dependent steps
+// is a sixteenth as long. With b_t the sum of the chunk's log decays up to and including token t (per
+// key channel) and B = b of its last token:
 //
 //   o_t = qscale * ( (q_t * exp(b_t))^T S_prev + sum_{s <= t} A[t][s] v_s ),   A[t][s] = sum_d q_td k_sd exp(b_td - b_sd)
 //   S   = diag(exp(B)) S_prev + sum_s (k_s * exp(B - b_s)) v_s^T
 //
 // Every exponent is <= 0 (a decay never grows), whatever the decays are: the pair (t, s) gets its own
-// exponentials instead of a product of two factors that could overflow. Same block shape and state
-// layout as gla_scan; q, k and b of the chunk lie in LDS (dynamic: 3 * 16 * dk floats).
+// exponentials instead of a product of two factors that could overflow. A does not depend on the
+// state, so a kernel of its own makes it for all chunks of the step at once (gla_pairs: a block per
+// chunk and head); the kernel that walks the chunks (gla_chunk: a block per request, head and 64
+// columns of the state, a wave per 16 columns) is left with three small matrix products per chunk.
+// Chunks are counted from the first token that the request brings in this step.
 constexpr int kChunk = 16;
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-template <int DR>
+// pairs[token][head][16]: row (token - its chunk's first) of the chunk's A, zero beyond the diagonal.
+__global__ __launch_bounds__(kThreads) void gla_pairs_kernel(
+    const float* __restrict__ x, float* __restrict__ pairs, const int* __restrict__ q_start, int heads, int dk, int dv) {
+  extern __shared__ float pair_lds[];
+  float* qs = pair_lds;
+  float* ks = qs + kChunk * dk;
+  float* bs = ks + kChunk * dk;
+  const int s = blockIdx.z, hd = blockIdx.y, tid = threadIdx.x, w = tid >> 6, lane = tid & 63;
+  const int t0 = q_start[s] + blockIdx.x * kChunk, t_end = q_start[s + 1];
+  if (t0 >= t_end) return;
+  const int nc = min(kChunk, t_end - t0);
+  const int hk = heads * dk, hv = heads * dv, width = 3 * hk + 2 * hv;
+  for (int i = tid; i < nc * dk; i += kThreads) {
+    const int t = i / dk, d = i % dk;
+    const float* xr = x + static_cast<size_t>(t0 + t) * width + hd * dk + d;
+    qs[i] = xr[0];
+    ks[i] = xr[hk];
+    bs[i] = xr[2 * hk];
+  }
+  __syncthreads();
+  for (int d = tid; d < dk; d += kThreads)
+    for (int t = 1; t < nc; ++t) bs[t * dk + d] += bs[(t - 1) * dk + d];
+  __syncthreads();
+  for (int p = w; p < nc * kChunk; p += 4) {  // a wave a pair, its lanes over the key channels
+    const int t = p / kChunk, sidx = p % kChunk;
+    float a = 0.f;
+    if (sidx <= t) {
+      for (int d = lane; d < dk; d += kWave)
+        a = fmaf(qs[t * dk + d] * ks[sidx * dk + d], expf(bs[t * dk + d] - bs[sidx * dk + d]), a);
+      a = wave_sum(a);
+    }
+    if (lane == 0) pairs[(static_cast<size_t>(t0 + t) * heads + hd) * kChunk + sidx] = a;
+  }
+}
+
+// DT: tiles of 16 rows of the state (dk <= 16 DT; the rows beyond dk are zeros and stay so).
+// Wave w owns columns 16 w .. 16 w + 15 of the block's 64 and keeps their dk rows in the layout of
+// the instruction's result: lane (g = lane / 16, c = lane % 16) holds rows 16 j + 4 g + i (i < 4) of
+// column c in S[j][i]. The sums over the rows take them in the order i, then g, so that a lane's own
+// S[j][i] is the operand it has to supply; the sums over the chunk's tokens take token 4 g + i in step i.
+template <int DT>
 __global__ __launch_bounds__(kThreads) void gla_chunk_kernel(
-    const float* __restrict__ x, float* __restrict__ state, float* __restrict__ o, const int* __restrict__ q_start,
-    const int* __restrict__ state_slots, int heads, int dk, int dv, float qscale) {
-  extern __shared__ float chunk_lds[];
-  float* qs = chunk_lds;               // [kChunk][dk]: q, later q * exp(b)
-  float* ks = qs + kChunk * dk;        // [kChunk][dk]: k, later k * exp(B - b)
-  float* bs = ks + kChunk * dk;        // [kChunk][dk]: log decays, then their running sums
-  __shared__ float vs[kChunk][kWave];
-  __shared__ float A[kChunk][kChunk + 1];
-  __shared__ float red[4][kChunk][kWave];
+    const float* __restrict__ x, const float* __restrict__ pairs, float* __restrict__ state, float* __restrict__ o,
+    const int* __restrict__ q_start, const int* __restrict__ state_slots, int heads, int dk, int dv, float qscale) {
+  constexpr int dkp = 16 * DT, kQLd = dkp + 4, kTLd = kChunk + 4;
+  extern __shared__ __attribute__((aligned(16))) float chunk_lds[];
+  float* qd = chunk_lds;                 // [kChunk][kQLd]: q * exp(b)
+  float* kdt = qd + kChunk * kQLd;       // [dkp][kTLd]:    k * exp(B - b), transposed
+  float* bs = kdt + dkp * kTLd;          // [kChunk][dkp]:  running sums of the log decays
+  float* vt = bs + kChunk * dkp;         // [64][kTLd]:     v, transposed
+  float* am = vt + kWave * kTLd;         // [kChunk][kTLd]: A
+  float* eb = am + kChunk * kTLd;        // [dkp]:          exp(B)
   const int s = blockIdx.x, hd = blockIdx.y, tid = threadIdx.x, w = tid >> 6, lane = tid & 63;
-  const int col = blockIdx.z * kWave + lane;
+  const int g = lane >> 4, c = lane & 15;
+  const int col = blockIdx.z * kWave + 16 * w + c;
   const bool has_col = col < dv;
   const int t_begin = q_start[s], t_end = q_start[s + 1];
   const int hk = heads * dk, hv = heads * dv, width = 3 * hk + 2 * hv;
   float* st = state + (static_cast<size_t>(state_slots[s]) * heads + hd) * dk * dv;
-  float S[DR];
+  f32x4 S[DT];
 #pragma unroll
-  for (int r = 0; r < DR; ++r) {
-    const int row = w + 4 * r;
-    S[r] = has_col && row < dk ? st[static_cast<size_t>(row) * dv + col] : 0.f;
-  }
+  for (int j = 0; j < DT; ++j)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 16 * j + 4 * g + i;
+      S[j][i] = has_col && row < dk ? st[static_cast<size_t>(row) * dv + col] : 0.f;
+    }
   for (int t0 = t_begin; t0 < t_end; t0 += kChunk) {
     const int nc = min(kChunk, t_end - t0);
-    for (int i = tid; i < nc * dk; i += kThreads) {
-      const int t = i / dk, d = i % dk;
-      const float* xr = x + static_cast<size_t>(t0 + t) * width + hd * dk + d;
-      qs[i] = xr[0];
-      ks[i] = xr[hk];
-      bs[i] = xr[2 * hk];
+    __syncthreads();  // the previous chunk's LDS is read
+    for (int i = tid; i < kChunk * dkp; i += kThreads) {
+      const int t = i / dkp, d = i % dkp;
+      bs[i] = t < nc && d < dk ? x[static_cast<size_t>(t0 + t) * width + 2 * hk + hd * dk + d] : 0.f;
     }
-    for (int i = tid; i < nc * kWave; i += kThreads) {
-      const int t = i >> 6, c = blockIdx.z * kWave + (i & 63);
-      vs[t][i & 63] = c < dv ? x[static_cast<size_t>(t0 + t) * width + 3 * hk + hd * dv + c] : 0.f;
+    for (int i = tid; i < kChunk * kWave; i += kThreads) {
+      const int t = i >> 6, cc = i & 63, gc = blockIdx.z * kWave + cc;
+      vt[cc * kTLd + t] = t < nc && gc < dv ? x[static_cast<size_t>(t0 + t) * width + 3 * hk + hd * dv + gc] : 0.f;
     }
-    __syncthreads();
-    for (int d = tid; d < dk; d += kThreads)
-      for (int t = 1; t < nc; ++t) bs[t * dk + d] += bs[(t - 1) * dk + d];
-    __syncthreads();
-    // A[t][s] for s <= t: a wave a pair, its lanes over the key channels
-    for (int p = w; p < nc * (nc + 1) / 2; p += 4) {
-      int t = 0;
-      while ((t + 1) * (t + 2) / 2 <= p) ++t;
-      const int sidx = p - t * (t + 1) / 2;
-      float a = 0.f;
-      for (int d = lane; d < dk; d += kWave)
-        a = fmaf(qs[t * dk + d] * ks[sidx * dk + d], expf(bs[t * dk + d] - bs[sidx * dk + d]), a);
-      a = wave_sum(a);
-      if (lane == 0) A[t][sidx] = a;
+    {
+      const int t = tid >> 4, sidx = tid & 15;
+      am[t * kTLd + sidx] = t < nc && sidx <= t ? pairs[(static_cast<size_t>(t0 + t) * heads + hd) * kChunk + sidx] : 0.f;
     }
     __syncthreads();
-    for (int i = tid; i < nc * dk; i += kThreads) {
-      const int d = i % dk;
-      qs[i] *= expf(bs[i]);
-      ks[i] *= expf(bs[(nc - 1) * dk + d] - bs[i]);
+    for (int d = tid; d < dkp; d += kThreads) {
+      for (int t = 1; t < nc; ++t) bs[t * dkp + d] += bs[(t - 1) * dkp + d];
+      eb[d] = expf(bs[(nc - 1) * dkp + d]);
     }
     __syncthreads();
-    for (int t = 0; t < nc; ++t) {
-      float part = 0.f;
-#pragma unroll
-      for (int r = 0; r < DR; ++r) {
-        const int row = w + 4 * r;
-        if (row < dk) part = fmaf(S[r], qs[t * dk + row], part);
+    for (int i = tid; i < kChunk * dkp; i += kThreads) {
+      const int t = i / dkp, d = i % dkp;
+      float qv = 0.f, kv = 0.f;
+      if (t < nc && d < dk) {
+        const float* xr = x + static_cast<size_t>(t0 + t) * width + hd * dk + d;
+        qv = xr[0] * expf(bs[i]);
+        kv = xr[hk] * expf(bs[(nc - 1) * dkp + d] - bs[i]);
       }
-      red[w][t][lane] = part;
-    }
-#pragma unroll
-    for (int r = 0; r < DR; ++r) {
-      const int row = w + 4 * r;
-      if (row < dk) {
-        float add = 0.f;
-        for (int t = 0; t < nc; ++t) add = fmaf(ks[t * dk + row], vs[t][lane], add);
-        S[r] = expf(bs[(nc - 1) * dk + row]) * S[r] + add;
-      }
+      qd[t * kQLd + d] = qv;
+      kdt[d * kTLd + t] = kv;
     }
     __syncthreads();
-    for (int t = w; t < nc; t += 4) {
-      float acc = ((red[0][t][lane] + red[1][t][lane]) + red[2][t][lane]) + red[3][t][lane];
-      for (int sidx = 0; sidx <= t; ++sidx) acc = fmaf(A[t][sidx], vs[sidx][lane], acc);
-      if (has_col) o[static_cast<size_t>(t0 + t) * hv + hd * dv + col] = acc * qscale;
+    // this wave's 16 columns: lane (g, c) takes tokens 4 g + i of the results, token row c of the operands
+    const f32x4 v4 = *reinterpret_cast<const f32x4*>(&vt[(16 * w + c) * kTLd + 4 * g]);
+    f32x4 out = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < DT; ++j) {
+      const f32x4 q4 = *reinterpret_cast<const f32x4*>(&qd[c * kQLd + 16 * j + 4 * g]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) out = __builtin_amdgcn_mfma_f32_16x16x4f32(q4[i], S[j][i], out, 0, 0, 0);
     }
-    __syncthreads();  // the chunk's LDS is read; the next chunk may load
+    {
+      const f32x4 a4 = *reinterpret_cast<const f32x4*>(&am[c * kTLd + 4 * g]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) out = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[i], v4[i], out, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int t = 4 * g + i;
+      if (t < nc && has_col) o[static_cast<size_t>(t0 + t) * hv + hd * dv + col] = out[i] * qscale;
+    }
+#pragma unroll
+    for (int j = 0; j < DT; ++j) {
+      const f32x4 e4 = *reinterpret_cast<const f32x4*>(&eb[16 * j + 4 * g]);
+      const f32x4 k4 = *reinterpret_cast<const f32x4*>(&kdt[(16 * j + c) * kTLd + 4 * g]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) S[j][i] *= e4[i];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) S[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(k4[i], v4[i], S[j], 0, 0, 0);
+    }
   }
 #pragma unroll
-  for (int r = 0; r < DR; ++r) {
-    const int row = w + 4 * r;
-    if (has_col && row < dk) st[static_cast<size_t>(row) * dv + col] = S[r];
-  }
+  for (int j = 0; j < DT; ++j)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 16 * j + 4 * g + i;
+      if (has_col && row < dk) st[static_cast<size_t>(row) * dv + col] = S[j][i];
+    }
 }
 
 __global__ __launch_bounds__(kThreads) void gla_finish_kernel(
@@ -261,19 +313,35 @@ extern "C" int pyre_gla_scan(const float* x, float* state, float* o, const int* 
   return check_launch("gla_scan");
 }
 
-extern "C" int pyre_gla_chunks(const float* x, float* state, float* o, const int* q_start, const int* state_slots,
-                               int n_seqs, int heads, int dk, int dv, float qscale, hipStream_t stream) {
+extern "C" int pyre_gla_chunks(const float* x, float* pairs, float* state, float* o, const int* q_start,
+                               const int* state_slots, int n_seqs, int max_tokens, int heads, int dk, int dv, float qscale,
+                               hipStream_t stream) {
   PYRE_REQUIRE(heads > 0 && heads <= 65535 && dk > 0 && dk <= 256 && dv > 0, "gla_chunks: heads %d, sizes %d / %d are not taken", heads, dk, dv);
-  if (n_seqs <= 0) return 0;
+  PYRE_REQUIRE(n_seqs <= 65535 && max_tokens >= 0, "gla_chunks: %d requests are more than a launch takes", n_seqs);
+  if (n_seqs <= 0 || max_tokens == 0) return 0;
+  hipLaunchKernelGGL(gla_pairs_kernel, dim3((max_tokens + kChunk - 1) / kChunk, heads, n_seqs), dim3(kThreads),
+                     sizeof(float) * 3 * kChunk * dk, stream, x, pairs, q_start, heads, dk, dv);
+  if (check_launch("gla_pairs")) return 1;
   const dim3 grid(n_seqs, heads, (dv + kWave - 1) / kWave);
-  const size_t lds = sizeof(float) * 3 * kChunk * dk;
-#define PYRE_CHUNKS(DR)                                                                                              \
-  hipLaunchKernelGGL(gla_chunk_kernel<DR>, grid, dim3(kThreads), lds, stream, x, state, o, q_start, state_slots, heads, \
-                     dk, dv, qscale)
-  if (dk <= 32) PYRE_CHUNKS(8);
-  else if (dk <= 64) PYRE_CHUNKS(16);
-  else if (dk <= 128) PYRE_CHUNKS(32);
-  else PYRE_CHUNKS(64);
+#define PYRE_CHUNKS(DT)                                                                                               \
+  do {                                                                                                                \
+    constexpr int dkp = 16 * DT;                                                                                      \
+    const size_t lds = sizeof(float) * (kChunk * (dkp + 4) + dkp * (kChunk + 4) + kChunk * dkp + kWave * (kChunk + 4) + \
+                                        kChunk * (kChunk + 4) + dkp);                                                 \
+    static bool raised = false;                                                                                       \
+    if (lds > 64 * 1024 && !raised) {                                                                                 \
+      PYRE_REQUIRE(hipFuncSetAttribute(reinterpret_cast<const void*>(&gla_chunk_kernel<DT>),                          \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) == hipSuccess, \
+                   "gla_chunks: the device refuses %zu bytes of LDS", lds);                                          \
+      raised = true;                                                                                                  \
+    }                                                                                                                 \
+    hipLaunchKernelGGL(gla_chunk_kernel<DT>, grid, dim3(kThreads), lds, stream, x, pairs, state, o, q_start,          \
+                       state_slots, heads, dk, dv, qscale);                                                           \
+  } while (0)
+  if (dk <= 32) PYRE_CHUNKS(2);
+  else if (dk <= 64) PYRE_CHUNKS(4);
+  else if (dk <= 128) PYRE_CHUNKS(8);
+  else PYRE_CHUNKS(16);
 #undef PYRE_CHUNKS
   return check_launch("gla_chunks");
 }

@@ -329,19 +329,28 @@ def gla_prepare(proj: Partials, col0: int, a2: torch.Tensor, a2_bias: torch.Tens
 
 
 def gla_scan(x: torch.Tensor, state: torch.Tensor, o: torch.Tensor, q_start: torch.Tensor, state_slots: torch.Tensor,
-             n_seqs: int, heads: int, dk: int, dv: int, qscale: float, chunks: bool = False) -> None:
+             n_seqs: int, heads: int, dk: int, dv: int, qscale: float, chunks: torch.Tensor | None = None,
+             max_tokens: int = 0) -> None:
     """The recurrence over each request's tokens of the step, from and into ``state [slots, heads, dk, dv]``;
-    ``o`` (float32 [N, heads*dv]) receives qscale * S^T q. ``chunks``: sixteen tokens at a time (for steps
-    that carry prompt portions; the token-by-token walk is the one for single tokens), a difference of rounding."""
-    _dev(x, state, o, q_start, state_slots)
+    ``o`` (float32 [N, heads*dv]) receives qscale * S^T q. ``chunks``: scratch (float32, 16 per token and head)
+    that makes the walk take sixteen tokens at a time on the matrix cores (for steps that carry prompt portions,
+    ``max_tokens`` the most that one request brings; the token-by-token walk is the one for single tokens): a
+    difference of rounding."""
+    _dev(x, state, o, q_start, state_slots, chunks)
     for name, t in (("x", x), ("state", state), ("o", o)):
         if t.dtype != torch.float32 or not t.is_contiguous():
             raise KernelError(f"gla_scan: {name} is contiguous float32")
     if tuple(state.shape[1:]) != (heads, dk, dv) or x.shape[-1] != gla_row_width(heads, dk, dv) or o.shape[-1] != heads * dv:
         raise KernelError("gla_scan: shapes do not fit the head geometry")
     _i32("q_start", q_start, n_seqs + 1), _i32("state_slots", state_slots, n_seqs)
-    call("pyre_gla_chunks" if chunks else "pyre_gla_scan", x.data_ptr(), state.data_ptr(), o.data_ptr(), q_start.data_ptr(), state_slots.data_ptr(),
-         n_seqs, heads, dk, dv, float(qscale), _stream())
+    if chunks is None:
+        call("pyre_gla_scan", x.data_ptr(), state.data_ptr(), o.data_ptr(), q_start.data_ptr(), state_slots.data_ptr(),
+             n_seqs, heads, dk, dv, float(qscale), _stream())
+        return
+    if chunks.dtype != torch.float32 or not chunks.is_contiguous() or chunks.numel() < x.shape[0] * heads * 16:
+        raise KernelError("gla_scan: the chunks' scratch is contiguous float32, 16 per token and head")
+    call("pyre_gla_chunks", x.data_ptr(), chunks.data_ptr(), state.data_ptr(), o.data_ptr(), q_start.data_ptr(),
+         state_slots.data_ptr(), n_seqs, int(max_tokens), heads, dk, dv, float(qscale), _stream())
 
 
 def gla_finish(o: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: float, out_scale: float, out: torch.Tensor,
