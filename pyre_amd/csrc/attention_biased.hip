@@ -85,6 +85,21 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 constexpr int kKeys = 32;
 constexpr int kTileMaxKeyHead = 128;  // the queries of a block's four heads lie in LDS
 
+// Eight consecutive elements as floats in one or two 16-byte loads; p is aligned to 16 bytes.
+__device__ inline void load8(const float* p, float (&v)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+}
+__device__ inline void load8(const bf16* p, float (&v)[8]) {
+  const uint4 r = *reinterpret_cast<const uint4*>(p);
+  const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    v[2 * u] = __uint_as_float(w[u] << 16);
+    v[2 * u + 1] = __uint_as_float(w[u] & 0xffff0000u);
+  }
+}
+
 __device__ inline float shaped_score(float raw, float scale, float cap, const float* bias_row, int dist, int far) {
   float s = raw * scale;
   if (cap > 0.f) s = cap * tanhf(s / cap);
@@ -96,7 +111,9 @@ __device__ inline float shaped_score(float raw, float scale, float cap, const fl
 // size is a run-time number of up to 128, padded to a multiple of 32 in LDS. Layout as in attention_f32_mfma.hip:
 // the transposed problem, S^T[key, token] and O^T[d, token], so that a lane's sixteen scores are
 // the operands of the second product as they are.
-template <typename T, int NV>
+// VEC: both head sizes are multiples of eight and the caches start on 16 bytes, so that keys and
+// values come eight elements to a load.
+template <typename T, int NV, bool VEC>
 __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, T* __restrict__ out,
     int out_ld, const float* __restrict__ gate, float out_scale, const int* __restrict__ tiles,
@@ -155,19 +172,39 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
       page_s[tid] = key <= hi_all && entry < table_stride ? table[entry] : -1;
     }
     __syncthreads();
-    for (int i = tid; i < kKeys * dkp; i += kThreads) {
-      const int key = i / dkp, d = i % dkp, page = page_s[key];
-      float v = 0.f;
-      if (page >= 0 && d < dk)
-        v = to_float(k_cache[((static_cast<size_t>(page) * nkv + kvh) * page_size + (key0 + key) % page_size) * dk + d]);
-      Ks[key * ldk + d] = v;
-    }
-    for (int i = tid; i < kKeys * 32 * NV; i += kThreads) {
-      const int key = i / (32 * NV), d = i % (32 * NV), page = page_s[key];
-      float v = 0.f;
-      if (page >= 0 && d < dv)
-        v = to_float(v_cache[((static_cast<size_t>(page) * nkv + kvh) * page_size + (key0 + key) % page_size) * dv + d]);
-      Vt[d * (kKeys + 1) + key] = v;
+    if (VEC) {
+      const int kg = dkp / 8;
+      for (int i = tid; i < kKeys * kg; i += kThreads) {
+        const int key = i / kg, d = 8 * (i % kg), page = page_s[key];
+        float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (page >= 0 && d < dk)
+          load8(k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + (key0 + key) % page_size) * dk + d, v);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) Ks[key * ldk + d + u] = v[u];
+      }
+      for (int i = tid; i < kKeys * 4 * NV; i += kThreads) {
+        const int key = i / (4 * NV), d = 8 * (i % (4 * NV)), page = page_s[key];
+        float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (page >= 0 && d < dv)
+          load8(v_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + (key0 + key) % page_size) * dv + d, v);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) Vt[(d + u) * (kKeys + 1) + key] = v[u];
+      }
+    } else {
+      for (int i = tid; i < kKeys * dkp; i += kThreads) {
+        const int key = i / dkp, d = i % dkp, page = page_s[key];
+        float v = 0.f;
+        if (page >= 0 && d < dk)
+          v = to_float(k_cache[((static_cast<size_t>(page) * nkv + kvh) * page_size + (key0 + key) % page_size) * dk + d]);
+        Ks[key * ldk + d] = v;
+      }
+      for (int i = tid; i < kKeys * 32 * NV; i += kThreads) {
+        const int key = i / (32 * NV), d = i % (32 * NV), page = page_s[key];
+        float v = 0.f;
+        if (page >= 0 && d < dv)
+          v = to_float(v_cache[((static_cast<size_t>(page) * nkv + kvh) * page_size + (key0 + key) % page_size) * dv + d]);
+        Vt[d * (kKeys + 1) + key] = v;
+      }
     }
     __syncthreads();
     if (!active) continue;
@@ -231,14 +268,15 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
 constexpr int kSpan = 128;
 constexpr int kMaxHead = 256;
 
-template <typename T>
+// VEC: the key head is a multiple of eight elements and the cache starts on 16 bytes (a key in 16-byte loads).
+template <typename T, bool VEC>
 __global__ __launch_bounds__(kThreads) void attn_biased_single_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, T* __restrict__ out,
     int out_ld, const float* __restrict__ gate, float out_scale, const int* __restrict__ tokens,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale, float cap,
     const float* __restrict__ bias, int far, int window, int keep_first) {
-  __shared__ float qs[kMaxHead];
+  __shared__ __attribute__((aligned(16))) float qs[kMaxHead];
   __shared__ float sc[kSpan];
   __shared__ float accs[kThreads];
   __shared__ float scratch[16];
@@ -268,7 +306,17 @@ __global__ __launch_bounds__(kThreads) void attn_biased_single_kernel(
       if (page >= 0) {
         const T* kp = k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + off) * dk;
         s = 0.f;
-        for (int e = 0; e < dk; ++e) s = fmaf(qs[e], to_float(kp[e]), s);
+        if (VEC) {
+#pragma unroll 4
+          for (int e = 0; e < dk; e += 8) {
+            float kv[8];
+            load8(kp + e, kv);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s = fmaf(qs[e + u], kv[u], s);
+          }
+        } else {
+          for (int e = 0; e < dk; ++e) s = fmaf(qs[e], to_float(kp[e]), s);
+        }
         s = shaped_score(s, scale, cap, bias_row, pos - key, far);
       }
       sc[j] = s;
@@ -348,28 +396,34 @@ extern "C" int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int d
   const int nvp = nv <= 1 ? 1 : nv <= 2 ? 2 : nv <= 4 ? 4 : 8;
   const size_t lds = sizeof(float) * (static_cast<size_t>(kKeys + 4 * 32) * (dkp + 1) + 32 * nvp * (kKeys + 1));
   const dim3 grid(n_tiles, nkv * hgroups);
-#define PYRE_TILE(T, NV)                                                                                             \
+#define PYRE_TILE(T, NV, VEC)                                                                                           \
   do {                                                                                                               \
     static size_t raised = 64 * 1024;                                                                                \
     if (lds > raised) {                                                                                              \
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_biased_tile_kernel<T, NV>),                        \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_biased_tile_kernel<T, NV, VEC>),                        \
                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess)      \
         return fail("attn_biased_tile: the device refuses %zu bytes of LDS", lds);                                   \
       raised = lds;                                                                                                  \
     }                                                                                                                \
-    hipLaunchKernelGGL((attn_biased_tile_kernel<T, NV>), grid, dim3(kThreads), lds, stream, static_cast<const T*>(q), \
+    hipLaunchKernelGGL((attn_biased_tile_kernel<T, NV, VEC>), grid, dim3(kThreads), lds, stream, static_cast<const T*>(q), \
                        static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), static_cast<T*>(out), out_ld, \
                        gate, out_scale, tiles, positions, seq_of_token, block_table, table_stride, nq, nkv, dk, dkp,  \
                        dv, page_size, scale, cap, bias, far, window, keep_first);                                    \
   } while (0)
-#define PYRE_TILE_NV(T)                \
-  switch (nvp) {                       \
-    case 1: PYRE_TILE(T, 1); break;    \
-    case 2: PYRE_TILE(T, 2); break;    \
-    case 4: PYRE_TILE(T, 4); break;    \
-    default: PYRE_TILE(T, 8); break;   \
+#define PYRE_TILE_NV(T, VEC)                \
+  switch (nvp) {                            \
+    case 1: PYRE_TILE(T, 1, VEC); break;    \
+    case 2: PYRE_TILE(T, 2, VEC); break;    \
+    case 4: PYRE_TILE(T, 4, VEC); break;    \
+    default: PYRE_TILE(T, 8, VEC); break;   \
   }
-  if (dt == kF32) { PYRE_TILE_NV(float) } else { PYRE_TILE_NV(bf16) }
+  const bool vec = dk % 8 == 0 && dv % 8 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(v_cache) % 16 == 0;
+  if (dt == kF32) {
+    if (vec) { PYRE_TILE_NV(float, true) } else { PYRE_TILE_NV(float, false) }
+  } else {
+    if (vec) { PYRE_TILE_NV(bf16, true) } else { PYRE_TILE_NV(bf16, false) }
+  }
 #undef PYRE_TILE_NV
 #undef PYRE_TILE
   return check_launch("attn_biased_tile");
@@ -384,10 +438,17 @@ extern "C" int pyre_attn_biased_single(const void* q, void* out, int out_ld, int
   if (check_geometry("attn_biased_single", nq, nkv, dk, dv, page_size)) return 1;
   PYRE_REQUIRE(known_dtype(dt) && table_stride > 0 && window >= 0 && keep_first >= 0 && far >= 0, "attn_biased_single: bad arguments");
   if (n <= 0) return 0;
-  PYRE_DISPATCH(dt, T,
-      hipLaunchKernelGGL(attn_biased_single_kernel<T>, dim3(n, nq), dim3(kThreads), 0, stream, static_cast<const T*>(q),
-                         static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), static_cast<T*>(out), out_ld,
-                         gate, out_scale, tokens, positions, seq_of_token, block_table, table_stride, nq, nkv, dk, dv,
-                         page_size, scale, cap, bias, far, window, keep_first));
+#define PYRE_SINGLE(VEC)                                                                                                 \
+  PYRE_DISPATCH(dt, T,                                                                                                    \
+      hipLaunchKernelGGL((attn_biased_single_kernel<T, VEC>), dim3(n, nq), dim3(kThreads), 0, stream,                     \
+                         static_cast<const T*>(q), static_cast<const T*>(k_cache), static_cast<const T*>(v_cache),        \
+                         static_cast<T*>(out), out_ld, gate, out_scale, tokens, positions, seq_of_token, block_table,     \
+                         table_stride, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first))
+  if (dk % 8 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0) {
+    PYRE_SINGLE(true);
+  } else {
+    PYRE_SINGLE(false);
+  }
+#undef PYRE_SINGLE
   return check_launch("attn_biased_single");
 }

@@ -13,6 +13,7 @@
 // With `rows` only the listed rows are normed, into out[0 .. n), and resid is left as it was.
 #include "pyre_api.h"
 #include "pyre_common.h"
+#include "pyre_vec4.h"
 
 using namespace pyre;
 
@@ -116,6 +117,29 @@ __global__ void clipped_glu_kernel(const void* __restrict__ gu, int gu_dt, int n
   store_from_float(out, out_dt, i, g / (1.f + expf(-slope * g)) * (u + 1.f));
 }
 
+__device__ inline float clipped_unit(float g, float u, float limit, float slope) {
+  if (limit > 0.f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+  }
+  return g / (1.f + expf(-slope * g)) * (u + 1.f);
+}
+
+// The same, four elements a thread (inter and the partial sums' stride are multiples of four).
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void clipped_glu_vec_kernel(const TI* __restrict__ gu, int n_partials, size_t partial_stride,
+                                                              TO* __restrict__ out, size_t total4, int inter, float limit,
+                                                              float slope) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= total4) return;
+  const int per_row = inter / 4;
+  const size_t n = i / per_row, c = 4 * (i % per_row);
+  const size_t gi = n * 2 * inter + c;
+  const float4 g = sum_partials4(gu + gi, partial_stride, n_partials), u = sum_partials4(gu + gi + inter, partial_stride, n_partials);
+  Vec4<TO>::store(out + n * inter + c, float4{clipped_unit(g.x, u.x, limit, slope), clipped_unit(g.y, u.y, limit, slope),
+                                              clipped_unit(g.z, u.z, limit, slope), clipped_unit(g.w, u.w, limit, slope)});
+}
+
 __global__ void scale_kernel(float* __restrict__ x, size_t total, float s) {
   const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i < total) x[i] *= s;
@@ -155,6 +179,15 @@ extern "C" int pyre_clipped_glu(const void* gu, int gu_dt, int n_partials, long 
   PYRE_REQUIRE(known_dtype(gu_dt) && known_dtype(out_dt), "clipped_glu: unknown dtype");
   PYRE_REQUIRE(n_partials >= 1 && inter > 0, "clipped_glu: bad sizes");
   if (n <= 0) return 0;
+  if (inter % 4 == 0 && partial_stride % 4 == 0 && reinterpret_cast<uintptr_t>(gu) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+    const size_t total4 = static_cast<size_t>(n) * (inter / 4);
+    PYRE_DISPATCH(gu_dt, TI, PYRE_DISPATCH(out_dt, TO,
+        hipLaunchKernelGGL((clipped_glu_vec_kernel<TI, TO>), dim3((total4 + 255) / 256), dim3(256), 0, stream,
+                           static_cast<const TI*>(gu), n_partials, static_cast<size_t>(partial_stride),
+                           static_cast<TO*>(out), total4, inter, limit, slope)));
+    return check_launch("clipped_glu");
+  }
   const size_t total = static_cast<size_t>(n) * inter;
   hipLaunchKernelGGL(clipped_glu_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, gu, gu_dt, n_partials,
                      static_cast<size_t>(partial_stride), out, out_dt, total, inter, limit, slope);

@@ -100,34 +100,59 @@ __global__ __launch_bounds__(kThreads) void gla_scan_kernel(
   }
 }
 
-// The same recurrence for requests that bring many tokens: chunks of 16 tokens, each worked on by a
-// whole block at once on the matrix cores' float32 instruction, so that the chain of dependent steps
-// is a sixteenth as long. With b_t the sum of the chunk's log decays up to and including token t (per
-// key channel) and B = b of its last token:
+// The same recurrence for requests that bring many tokens: chunks of 16 tokens on the matrix cores'
+// float32 instruction, so that the chain of dependent steps is a sixteenth as long. With b_t the sum
+// of the chunk's log decays up to and including token t (per key channel) and B = b of its last token:
 //
 //   o_t = qscale * ( (q_t * exp(b_t))^T S_prev + sum_{s <= t} A[t][s] v_s ),   A[t][s] = sum_d q_td k_sd exp(b_td - b_sd)
 //   S   = diag(exp(B)) S_prev + sum_s (k_s * exp(B - b_s)) v_s^T
 //
 // Every exponent is <= 0 (a decay never grows), whatever the decays are: the pair (t, s) gets its own
-// exponentials instead of a product of two factors that could overflow. A does not depend on the
-// state, so a kernel of its own makes it for all chunks of the step at once (gla_pairs: a block per
-// chunk and head); the kernel that walks the chunks (gla_chunk: a block per request, head and 64
-// columns of the state, a wave per 16 columns) is left with three small matrix products per chunk.
-// Chunks are counted from the first token that the request brings in this step.
+// exponentials instead of a product of two factors that could overflow. Nothing but S_prev depends on
+// the chunks before, so one kernel prepares all chunks of the step at once (gla_chunk_prep: a block per
+// chunk and head makes A, q * exp(b), k * exp(B - b), exp(B) and v in the layouts of the matrix
+// instruction's operands) and the kernel that walks the chunks (gla_chunk_walk: a wave per request,
+// head and 16 columns of the state, nothing shared between waves) is left with three small matrix
+// products per chunk, whose operands it asks for one chunk ahead.
+// Chunks are counted from the first token that the request brings in this step. A chunk's operands
+// lie at "slots": token t of request s of the step has slot t + 16 s, so that the 16 slots of a
+// request's last, shorter chunk do not reach into the next request's.
 constexpr int kChunk = 16;
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-// pairs[token][head][16]: row (token - its chunk's first) of the chunk's A, zero beyond the diagonal.
-__global__ __launch_bounds__(kThreads) void gla_pairs_kernel(
-    const float* __restrict__ x, float* __restrict__ pairs, const int* __restrict__ q_start, int heads, int dk, int dv) {
-  extern __shared__ float pair_lds[];
-  float* qs = pair_lds;
+struct ChunkScratch {
+  float* qd;     // [slot][head][dkp]:                 q * exp(b)
+  float* kdt;    // per chunk [head][dkp][16 tokens]:  k * exp(B - b)
+  float* vt;     // per chunk [head][dvp][16 tokens]:  v
+  float* pairs;  // [slot][head][16]:                  row of A
+  float* eb;     // per chunk [head][256]:             exp(B)
+};
+__host__ __device__ inline size_t chunk_scratch_floats(size_t slots, int heads, int dkp, int dvp) {
+  return slots * heads * (2 * static_cast<size_t>(dkp) + dvp + 2 * kChunk);
+}
+__host__ __device__ inline ChunkScratch carve(float* base, size_t slots, int heads, int dkp, int dvp) {
+  ChunkScratch c;
+  c.qd = base;
+  c.kdt = c.qd + slots * heads * dkp;
+  c.vt = c.kdt + slots * heads * dkp;
+  c.pairs = c.vt + slots * heads * dvp;
+  c.eb = c.pairs + slots * heads * kChunk;
+  return c;
+}
+
+__global__ __launch_bounds__(kThreads) void gla_chunk_prep_kernel(
+    const float* __restrict__ x, ChunkScratch sc, const int* __restrict__ q_start, int heads, int dk, int dv, int dkp,
+    int dvp) {
+  extern __shared__ float prep_lds[];
+  float* qs = prep_lds;
   float* ks = qs + kChunk * dk;
   float* bs = ks + kChunk * dk;
   const int s = blockIdx.z, hd = blockIdx.y, tid = threadIdx.x, w = tid >> 6, lane = tid & 63;
   const int t0 = q_start[s] + blockIdx.x * kChunk, t_end = q_start[s + 1];
   if (t0 >= t_end) return;
   const int nc = min(kChunk, t_end - t0);
+  const size_t slot0 = static_cast<size_t>(t0) + kChunk * s;
+  const size_t region = slot0 * heads + static_cast<size_t>(hd) * kChunk;  // of this chunk and head, in slots
   const int hk = heads * dk, hv = heads * dv, width = 3 * hk + 2 * hv;
   for (int i = tid; i < nc * dk; i += kThreads) {
     const int t = i / dk, d = i % dk;
@@ -136,45 +161,56 @@ __global__ __launch_bounds__(kThreads) void gla_pairs_kernel(
     ks[i] = xr[hk];
     bs[i] = xr[2 * hk];
   }
+  for (int i = tid; i < dvp * kChunk; i += kThreads) {
+    const int cc = i / kChunk, t = i % kChunk;
+    sc.vt[region * dvp + i] = t < nc && cc < dv ? x[static_cast<size_t>(t0 + t) * width + 3 * hk + hd * dv + cc] : 0.f;
+  }
   __syncthreads();
   for (int d = tid; d < dk; d += kThreads)
     for (int t = 1; t < nc; ++t) bs[t * dk + d] += bs[(t - 1) * dk + d];
   __syncthreads();
-  for (int p = w; p < nc * kChunk; p += 4) {  // a wave a pair, its lanes over the key channels
+  for (int p = w; p < kChunk * kChunk; p += 4) {  // a wave a pair, its lanes over the key channels
     const int t = p / kChunk, sidx = p % kChunk;
     float a = 0.f;
-    if (sidx <= t) {
+    if (sidx <= t && t < nc) {
       for (int d = lane; d < dk; d += kWave)
         a = fmaf(qs[t * dk + d] * ks[sidx * dk + d], expf(bs[t * dk + d] - bs[sidx * dk + d]), a);
       a = wave_sum(a);
     }
-    if (lane == 0) pairs[(static_cast<size_t>(t0 + t) * heads + hd) * kChunk + sidx] = a;
+    if (lane == 0) sc.pairs[((slot0 + t) * heads + hd) * kChunk + sidx] = a;
   }
+  for (int i = tid; i < kChunk * dkp; i += kThreads) {
+    const int t = i / dkp, d = i % dkp;
+    const bool there = t < nc && d < dk;
+    sc.qd[((slot0 + t) * heads + hd) * dkp + d] = there ? qs[t * dk + d] * expf(bs[t * dk + d]) : 0.f;
+  }
+  for (int i = tid; i < kChunk * dkp; i += kThreads) {
+    const int d = i / kChunk, t = i % kChunk;
+    const bool there = t < nc && d < dk;
+    sc.kdt[region * dkp + i] = there ? ks[t * dk + d] * expf(bs[(nc - 1) * dk + d] - bs[t * dk + d]) : 0.f;
+  }
+  for (int d = tid; d < dkp; d += kThreads) sc.eb[region * kChunk + d] = d < dk ? expf(bs[(nc - 1) * dk + d]) : 0.f;
 }
 
-// DT: tiles of 16 rows of the state (dk <= 16 DT; the rows beyond dk are zeros and stay so).
-// Wave w owns columns 16 w .. 16 w + 15 of the block's 64 and keeps their dk rows in the layout of
-// the instruction's result: lane (g = lane / 16, c = lane % 16) holds rows 16 j + 4 g + i (i < 4) of
-// column c in S[j][i]. The sums over the rows take them in the order i, then g, so that a lane's own
-// S[j][i] is the operand it has to supply; the sums over the chunk's tokens take token 4 g + i in step i.
+// DT: tiles of 16 rows of the state (dk <= 16 DT; the rows beyond dk are zeros and stay so). The wave
+// keeps its 16 columns' rows in the layout of the instruction's result: lane (g = lane / 16,
+// c = lane % 16) holds rows 16 j + 4 g + i (i < 4) of column c in S[j][i]. The sums over the rows take
+// them in the order i, then g, so that a lane's own S[j][i] is the operand it has to supply; the sums
+// over the chunk's tokens take token 4 g + i in step i.
 template <int DT>
-__global__ __launch_bounds__(kThreads) void gla_chunk_kernel(
-    const float* __restrict__ x, const float* __restrict__ pairs, float* __restrict__ state, float* __restrict__ o,
-    const int* __restrict__ q_start, const int* __restrict__ state_slots, int heads, int dk, int dv, float qscale) {
-  constexpr int dkp = 16 * DT, kQLd = dkp + 4, kTLd = kChunk + 4;
-  extern __shared__ __attribute__((aligned(16))) float chunk_lds[];
-  float* qd = chunk_lds;                 // [kChunk][kQLd]: q * exp(b)
-  float* kdt = qd + kChunk * kQLd;       // [dkp][kTLd]:    k * exp(B - b), transposed
-  float* bs = kdt + dkp * kTLd;          // [kChunk][dkp]:  running sums of the log decays
-  float* vt = bs + kChunk * dkp;         // [64][kTLd]:     v, transposed
-  float* am = vt + kWave * kTLd;         // [kChunk][kTLd]: A
-  float* eb = am + kChunk * kTLd;        // [dkp]:          exp(B)
-  const int s = blockIdx.x, hd = blockIdx.y, tid = threadIdx.x, w = tid >> 6, lane = tid & 63;
-  const int g = lane >> 4, c = lane & 15;
-  const int col = blockIdx.z * kWave + 16 * w + c;
+struct ChunkOperands {
+  f32x4 q[DT], k[DT], e[DT], v, a;
+};
+
+template <int DT>
+__global__ __launch_bounds__(kWave) void gla_chunk_walk_kernel(
+    ChunkScratch sc, float* __restrict__ state, float* __restrict__ o, const int* __restrict__ q_start,
+    const int* __restrict__ state_slots, int heads, int dk, int dv, int dvp, float qscale) {
+  constexpr int dkp = 16 * DT;
+  const int s = blockIdx.x, hd = blockIdx.y, lane = threadIdx.x, g = lane >> 4, c = lane & 15;
+  const int col = blockIdx.z * 16 + c;
   const bool has_col = col < dv;
-  const int t_begin = q_start[s], t_end = q_start[s + 1];
-  const int hk = heads * dk, hv = heads * dv, width = 3 * hk + 2 * hv;
+  const int t_begin = q_start[s], t_end = q_start[s + 1], hv = heads * dv;
   float* st = state + (static_cast<size_t>(state_slots[s]) * heads + hd) * dk * dv;
   f32x4 S[DT];
 #pragma unroll
@@ -184,53 +220,35 @@ __global__ __launch_bounds__(kThreads) void gla_chunk_kernel(
       const int row = 16 * j + 4 * g + i;
       S[j][i] = has_col && row < dk ? st[static_cast<size_t>(row) * dv + col] : 0.f;
     }
-  for (int t0 = t_begin; t0 < t_end; t0 += kChunk) {
-    const int nc = min(kChunk, t_end - t0);
-    __syncthreads();  // the previous chunk's LDS is read
-    for (int i = tid; i < kChunk * dkp; i += kThreads) {
-      const int t = i / dkp, d = i % dkp;
-      bs[i] = t < nc && d < dk ? x[static_cast<size_t>(t0 + t) * width + 2 * hk + hd * dk + d] : 0.f;
-    }
-    for (int i = tid; i < kChunk * kWave; i += kThreads) {
-      const int t = i >> 6, cc = i & 63, gc = blockIdx.z * kWave + cc;
-      vt[cc * kTLd + t] = t < nc && gc < dv ? x[static_cast<size_t>(t0 + t) * width + 3 * hk + hd * dv + gc] : 0.f;
-    }
-    {
-      const int t = tid >> 4, sidx = tid & 15;
-      am[t * kTLd + sidx] = t < nc && sidx <= t ? pairs[(static_cast<size_t>(t0 + t) * heads + hd) * kChunk + sidx] : 0.f;
-    }
-    __syncthreads();
-    for (int d = tid; d < dkp; d += kThreads) {
-      for (int t = 1; t < nc; ++t) bs[t * dkp + d] += bs[(t - 1) * dkp + d];
-      eb[d] = expf(bs[(nc - 1) * dkp + d]);
-    }
-    __syncthreads();
-    for (int i = tid; i < kChunk * dkp; i += kThreads) {
-      const int t = i / dkp, d = i % dkp;
-      float qv = 0.f, kv = 0.f;
-      if (t < nc && d < dk) {
-        const float* xr = x + static_cast<size_t>(t0 + t) * width + hd * dk + d;
-        qv = xr[0] * expf(bs[i]);
-        kv = xr[hk] * expf(bs[(nc - 1) * dkp + d] - bs[i]);
-      }
-      qd[t * kQLd + d] = qv;
-      kdt[d * kTLd + t] = kv;
-    }
-    __syncthreads();
-    // this wave's 16 columns: lane (g, c) takes tokens 4 g + i of the results, token row c of the operands
-    const f32x4 v4 = *reinterpret_cast<const f32x4*>(&vt[(16 * w + c) * kTLd + 4 * g]);
-    f32x4 out = {0.f, 0.f, 0.f, 0.f};
+  auto fetch = [&](int t0, ChunkOperands<DT>& r) {
+    const size_t slot0 = static_cast<size_t>(t0) + kChunk * s;
+    const size_t region = slot0 * heads + static_cast<size_t>(hd) * kChunk;
+    const float* qp = sc.qd + ((slot0 + c) * heads + hd) * dkp + 4 * g;
+    const float* kp = sc.kdt + region * dkp + c * kChunk + 4 * g;
+    const float* ep = sc.eb + region * kChunk + 4 * g;
 #pragma unroll
     for (int j = 0; j < DT; ++j) {
-      const f32x4 q4 = *reinterpret_cast<const f32x4*>(&qd[c * kQLd + 16 * j + 4 * g]);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) out = __builtin_amdgcn_mfma_f32_16x16x4f32(q4[i], S[j][i], out, 0, 0, 0);
+      r.q[j] = *reinterpret_cast<const f32x4*>(qp + 16 * j);
+      r.k[j] = *reinterpret_cast<const f32x4*>(kp + 16 * j * kChunk);
+      r.e[j] = *reinterpret_cast<const f32x4*>(ep + 16 * j);
     }
-    {
-      const f32x4 a4 = *reinterpret_cast<const f32x4*>(&am[c * kTLd + 4 * g]);
+    r.v = *reinterpret_cast<const f32x4*>(sc.vt + region * dvp + static_cast<size_t>(min(col, dvp - 1)) * kChunk + 4 * g);
+    if (!has_col) r.v = f32x4{0.f, 0.f, 0.f, 0.f};
+    r.a = *reinterpret_cast<const f32x4*>(sc.pairs + ((slot0 + c) * heads + hd) * kChunk + 4 * g);
+  };
+  ChunkOperands<DT> now, next;
+  if (t_begin < t_end) fetch(t_begin, now);
+  for (int t0 = t_begin; t0 < t_end; t0 += kChunk) {
+    const int nc = min(kChunk, t_end - t0);
+    const bool more = t0 + kChunk < t_end;
+    if (more) fetch(t0 + kChunk, next);
+    f32x4 out = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < 4; ++i) out = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[i], v4[i], out, 0, 0, 0);
-    }
+    for (int j = 0; j < DT; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) out = __builtin_amdgcn_mfma_f32_16x16x4f32(now.q[j][i], S[j][i], out, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out = __builtin_amdgcn_mfma_f32_16x16x4f32(now.a[i], now.v[i], out, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int t = 4 * g + i;
@@ -238,13 +256,12 @@ __global__ __launch_bounds__(kThreads) void gla_chunk_kernel(
     }
 #pragma unroll
     for (int j = 0; j < DT; ++j) {
-      const f32x4 e4 = *reinterpret_cast<const f32x4*>(&eb[16 * j + 4 * g]);
-      const f32x4 k4 = *reinterpret_cast<const f32x4*>(&kdt[(16 * j + c) * kTLd + 4 * g]);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) S[j][i] *= e4[i];
+      for (int i = 0; i < 4; ++i) S[j][i] *= now.e[j][i];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) S[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(k4[i], v4[i], S[j], 0, 0, 0);
+      for (int i = 0; i < 4; ++i) S[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(now.k[j][i], now.v[i], S[j], 0, 0, 0);
     }
+    if (more) now = next;
   }
 #pragma unroll
   for (int j = 0; j < DT; ++j)
@@ -313,36 +330,37 @@ extern "C" int pyre_gla_scan(const float* x, float* state, float* o, const int* 
   return check_launch("gla_scan");
 }
 
-extern "C" int pyre_gla_chunks(const float* x, float* pairs, float* state, float* o, const int* q_start,
-                               const int* state_slots, int n_seqs, int max_tokens, int heads, int dk, int dv, float qscale,
-                               hipStream_t stream) {
+static int chunk_tiles(int dk) { return dk <= 32 ? 2 : dk <= 64 ? 4 : dk <= 128 ? 8 : 16; }
+
+// Floats of scratch that pyre_gla_chunks needs for a step of n_tokens tokens of n_seqs requests.
+extern "C" long pyre_gla_chunks_scratch(int n_tokens, int n_seqs, int heads, int dk, int dv) {
+  const size_t slots = static_cast<size_t>(n_tokens) + static_cast<size_t>(kChunk) * n_seqs;
+  return static_cast<long>(chunk_scratch_floats(slots, heads, 16 * chunk_tiles(dk), (dv + 3) / 4 * 4));
+}
+
+extern "C" int pyre_gla_chunks(const float* x, float* scratch, float* state, float* o, const int* q_start,
+                               const int* state_slots, int n_tokens, int n_seqs, int max_tokens, int heads, int dk, int dv,
+                               float qscale, hipStream_t stream) {
   PYRE_REQUIRE(heads > 0 && heads <= 65535 && dk > 0 && dk <= 256 && dv > 0, "gla_chunks: heads %d, sizes %d / %d are not taken", heads, dk, dv);
-  PYRE_REQUIRE(n_seqs <= 65535 && max_tokens >= 0, "gla_chunks: %d requests are more than a launch takes", n_seqs);
+  PYRE_REQUIRE(n_seqs <= 65535 && max_tokens >= 0 && n_tokens >= 0, "gla_chunks: %d requests are more than a launch takes", n_seqs);
+  PYRE_REQUIRE(reinterpret_cast<uintptr_t>(scratch) % 16 == 0, "gla_chunks: the scratch memory must start on 16 bytes");
   if (n_seqs <= 0 || max_tokens == 0) return 0;
-  hipLaunchKernelGGL(gla_pairs_kernel, dim3((max_tokens + kChunk - 1) / kChunk, heads, n_seqs), dim3(kThreads),
-                     sizeof(float) * 3 * kChunk * dk, stream, x, pairs, q_start, heads, dk, dv);
-  if (check_launch("gla_pairs")) return 1;
-  const dim3 grid(n_seqs, heads, (dv + kWave - 1) / kWave);
-#define PYRE_CHUNKS(DT)                                                                                               \
-  do {                                                                                                                \
-    constexpr int dkp = 16 * DT;                                                                                      \
-    const size_t lds = sizeof(float) * (kChunk * (dkp + 4) + dkp * (kChunk + 4) + kChunk * dkp + kWave * (kChunk + 4) + \
-                                        kChunk * (kChunk + 4) + dkp);                                                 \
-    static bool raised = false;                                                                                       \
-    if (lds > 64 * 1024 && !raised) {                                                                                 \
-      PYRE_REQUIRE(hipFuncSetAttribute(reinterpret_cast<const void*>(&gla_chunk_kernel<DT>),                          \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) == hipSuccess, \
-                   "gla_chunks: the device refuses %zu bytes of LDS", lds);                                          \
-      raised = true;                                                                                                  \
-    }                                                                                                                 \
-    hipLaunchKernelGGL(gla_chunk_kernel<DT>, grid, dim3(kThreads), lds, stream, x, pairs, state, o, q_start,          \
-                       state_slots, heads, dk, dv, qscale);                                                           \
-  } while (0)
-  if (dk <= 32) PYRE_CHUNKS(2);
-  else if (dk <= 64) PYRE_CHUNKS(4);
-  else if (dk <= 128) PYRE_CHUNKS(8);
-  else PYRE_CHUNKS(16);
-#undef PYRE_CHUNKS
+  const int DTs = chunk_tiles(dk), dkp = 16 * DTs, dvp = (dv + 3) / 4 * 4;
+  const ChunkScratch sc = carve(scratch, static_cast<size_t>(n_tokens) + static_cast<size_t>(kChunk) * n_seqs, heads, dkp, dvp);
+  hipLaunchKernelGGL(gla_chunk_prep_kernel, dim3((max_tokens + kChunk - 1) / kChunk, heads, n_seqs), dim3(kThreads),
+                     sizeof(float) * 3 * kChunk * dk, stream, x, sc, q_start, heads, dk, dv, dkp, dvp);
+  if (check_launch("gla_chunk_prep")) return 1;
+  const dim3 grid(n_seqs, heads, (dv + 15) / 16);
+#define PYRE_WALK(DT)                                                                                                  \
+  hipLaunchKernelGGL(gla_chunk_walk_kernel<DT>, grid, dim3(kWave), 0, stream, sc, state, o, q_start, state_slots, heads, \
+                     dk, dv, dvp, qscale)
+  switch (DTs) {
+    case 2: PYRE_WALK(2); break;
+    case 4: PYRE_WALK(4); break;
+    case 8: PYRE_WALK(8); break;
+    default: PYRE_WALK(16); break;
+  }
+#undef PYRE_WALK
   return check_launch("gla_chunks");
 }
 

@@ -255,9 +255,10 @@ int pyre_gla_prepare(const void* proj, int proj_dt, int n_partials, long partial
 int pyre_gla_scan(const float* x, float* state, float* o, const int* q_start, const int* state_slots,
                   int n_seqs, int heads, int dk, int dv, float qscale, hipStream_t stream);
 // The same recurrence in chunks of 16 tokens (steps that carry prompt portions); differs from the scan by rounding.
-// pairs: scratch of tokens * heads * 16 floats; max_tokens: the most tokens that one request brings.
-int pyre_gla_chunks(const float* x, float* pairs, float* state, float* o, const int* q_start, const int* state_slots,
-                    int n_seqs, int max_tokens, int heads, int dk, int dv, float qscale, hipStream_t stream);
+// scratch: pyre_gla_chunks_scratch(...) floats, starting on 16 bytes; max_tokens: the most tokens that one request brings.
+long pyre_gla_chunks_scratch(int n_tokens, int n_seqs, int heads, int dk, int dv);
+int pyre_gla_chunks(const float* x, float* scratch, float* state, float* o, const int* q_start, const int* state_slots,
+                    int n_tokens, int n_seqs, int max_tokens, int heads, int dk, int dv, float qscale, hipStream_t stream);
 int pyre_gla_finish(const float* o, const float* x, const void* gain, int gain_dt, float eps, float out_scale,
                     void* out, int out_dt, int out_ld, int n, int heads, int dk, int dv, hipStream_t stream);
 

@@ -328,14 +328,23 @@ def gla_prepare(proj: Partials, col0: int, a2: torch.Tensor, a2_bias: torch.Tens
          dtype_code(a2_bias) if a2_bias is not None else 0, float(tau), x.data_ptr(), n, heads, dk, dv, rank, _stream())
 
 
+def gla_chunks_scratch(n_tokens: int, n_seqs: int, heads: int, dk: int, dv: int) -> int:
+    """Float32 elements of scratch that the walk in chunks needs for such a step."""
+    from pyre_amd.hip.lib import lib
+
+    fn = lib().pyre_gla_chunks_scratch
+    fn.restype = __import__("ctypes").c_long
+    return int(fn(n_tokens, n_seqs, heads, dk, dv))
+
+
 def gla_scan(x: torch.Tensor, state: torch.Tensor, o: torch.Tensor, q_start: torch.Tensor, state_slots: torch.Tensor,
              n_seqs: int, heads: int, dk: int, dv: int, qscale: float, chunks: torch.Tensor | None = None,
              max_tokens: int = 0) -> None:
     """The recurrence over each request's tokens of the step, from and into ``state [slots, heads, dk, dv]``;
-    ``o`` (float32 [N, heads*dv]) receives qscale * S^T q. ``chunks``: scratch (float32, 16 per token and head)
-    that makes the walk take sixteen tokens at a time on the matrix cores (for steps that carry prompt portions,
-    ``max_tokens`` the most that one request brings; the token-by-token walk is the one for single tokens): a
-    difference of rounding."""
+    ``o`` (float32 [N, heads*dv]) receives qscale * S^T q. ``chunks``: scratch (float32,
+    :func:`gla_chunks_scratch` elements) that makes the walk take sixteen tokens at a time on the matrix cores
+    (for steps that carry prompt portions, ``max_tokens`` the most that one request brings; the token-by-token
+    walk is the one for single tokens): a difference of rounding."""
     _dev(x, state, o, q_start, state_slots, chunks)
     for name, t in (("x", x), ("state", state), ("o", o)):
         if t.dtype != torch.float32 or not t.is_contiguous():
@@ -347,10 +356,11 @@ def gla_scan(x: torch.Tensor, state: torch.Tensor, o: torch.Tensor, q_start: tor
         call("pyre_gla_scan", x.data_ptr(), state.data_ptr(), o.data_ptr(), q_start.data_ptr(), state_slots.data_ptr(),
              n_seqs, heads, dk, dv, float(qscale), _stream())
         return
-    if chunks.dtype != torch.float32 or not chunks.is_contiguous() or chunks.numel() < x.shape[0] * heads * 16:
-        raise KernelError("gla_scan: the chunks' scratch is contiguous float32, 16 per token and head")
+    n = o.shape[0]
+    if chunks.dtype != torch.float32 or not chunks.is_contiguous() or chunks.numel() < gla_chunks_scratch(n, n_seqs, heads, dk, dv):
+        raise KernelError("gla_scan: the chunks' scratch is contiguous float32 of gla_chunks_scratch(...) elements")
     call("pyre_gla_chunks", x.data_ptr(), chunks.data_ptr(), state.data_ptr(), o.data_ptr(), q_start.data_ptr(),
-         state_slots.data_ptr(), n_seqs, int(max_tokens), heads, dk, dv, float(qscale), _stream())
+         state_slots.data_ptr(), n, n_seqs, int(max_tokens), heads, dk, dv, float(qscale), _stream())
 
 
 def gla_finish(o: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: float, out_scale: float, out: torch.Tensor,

@@ -67,7 +67,7 @@ class GatedLinearAttention(BranchMixer):
         # single tokens walk the recurrence as it is written; prompt portions take sixteen tokens at a time
         pairs = None
         if ctx.host.max_q_len > 1:
-            pairs = ws.get("gla.pairs", (n, s.num_heads, 16), torch.float32)
+            pairs = ws.get("gla.chunks", (ops.gla_chunks_scratch(n, ctx.n_seqs, *shape),), torch.float32)
         ops.gla_scan(x, cache.tensor, raw, ctx.q_start, cache.slots, ctx.n_seqs, *shape, s.key_dim ** -0.5,
                      chunks=pairs, max_tokens=ctx.host.max_q_len)
         ops.gla_finish(raw, x, self.gain, s.norm_eps, scale, o, n, *shape)
