@@ -278,6 +278,7 @@ __global__ __launch_bounds__(kThreads) void attn_biased_single_kernel(
     const float* __restrict__ bias, int far, int window, int keep_first) {
   __shared__ __attribute__((aligned(16))) float qs[kMaxHead];
   __shared__ float sc[kSpan];
+  __shared__ int row_s[kSpan];
   __shared__ float accs[kThreads];
   __shared__ float scratch[16];
   const int n = tokens ? tokens[blockIdx.x] : blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
@@ -303,6 +304,7 @@ __global__ __launch_bounds__(kThreads) void attn_biased_single_kernel(
       const int key = base + j;
       const int page = table[key / page_size], off = key % page_size;
       float s = -INFINITY;
+      row_s[j] = page >= 0 ? page * page_size + off : -1;  // the key's row in the cache, for the second product
       if (page >= 0) {
         const T* kp = k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + off) * dk;
         s = 0.f;
@@ -332,15 +334,25 @@ __global__ __launch_bounds__(kThreads) void attn_biased_single_kernel(
       sc[j] = p;
       lsum += p;
     }
-    l = l * alpha + block_sum(lsum, scratch);  // its barriers publish sc[]
+    l = l * alpha + block_sum(lsum, scratch);  // its barriers publish sc[] and row_s[]
     acc *= alpha;
-    if (active)
-      for (int j = g; j < cnt; j += groups) {
-        const int key = base + j;
-        const int page = table[key / page_size], off = key % page_size;
-        if (page < 0) continue;
-        acc = fmaf(sc[j], to_float(v_cache[((static_cast<size_t>(page) * nkv + kvh) * page_size + off) * dv + d]), acc);
+    if (active) {
+      // eight keys at a time, so that their values are on their way together
+      for (int j0 = g; j0 < cnt; j0 += 8 * groups) {
+        float vv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int j = j0 + u * groups;
+          const int row = j < cnt ? row_s[j] : -1;
+          vv[u] = row >= 0 ? to_float(v_cache[((static_cast<size_t>(row / page_size) * nkv + kvh) * page_size + row % page_size) * dv + d]) : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int j = j0 + u * groups;
+          if (j < cnt) acc = fmaf(sc[j], vv[u], acc);
+        }
       }
+    }
     __syncthreads();  // sc[] is read; the next span may write it
   }
   accs[tid] = active ? acc : 0.f;

@@ -96,6 +96,87 @@ __global__ __launch_bounds__(kThreads) void add_layernorm_kernel(
   }
 }
 
+// The same with four elements to a load (the row's width and the partial sums' stride are multiples
+// of four, no bias), the partial sums of an element asked for together: a step of few rows is all
+// waiting for loads. THREADS x ITEMS float4 hold a row.
+template <typename TD, typename TG, typename TO, int THREADS, int ITEMS>
+__global__ __launch_bounds__(THREADS) void add_layernorm_vec_kernel(
+    float* __restrict__ resid, const TD* __restrict__ delta, int n_partials, size_t partial_stride,
+    const TG* __restrict__ post_gain, const TG* __restrict__ post_scale, float post_eps, const TG* __restrict__ gain,
+    TO* __restrict__ out, const int* __restrict__ rows, int hidden, float eps) {
+  __shared__ float scratch[16];
+  const int r_out = blockIdx.x, r_in = rows ? rows[r_out] : r_out, tid = threadIdx.x, quads = hidden / 4;
+  const size_t row = static_cast<size_t>(r_in) * hidden;
+  const float inv_n = 1.f / static_cast<float>(hidden);
+  float4 v[ITEMS];
+  auto stats = [&](float e, float& mean, float& inv) {
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k)
+      if (tid + k * THREADS < quads) s += (v[k].x + v[k].y) + (v[k].z + v[k].w);
+    mean = block_sum(s, scratch) * inv_n;
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k)
+      if (tid + k * THREADS < quads) {
+        const float a = v[k].x - mean, b = v[k].y - mean, c = v[k].z - mean, d = v[k].w - mean;
+        ss += (a * a + b * b) + (c * c + d * d);
+      }
+    inv = 1.f / sqrtf(block_sum(ss, scratch) * inv_n + e);
+  };
+  if (delta) {
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+      const int i = 4 * (tid + k * THREADS);
+      v[k] = i < hidden ? sum_partials4(delta + row + i, partial_stride, n_partials) : float4{0.f, 0.f, 0.f, 0.f};
+    }
+    if (post_gain) {
+      float mean, inv;
+      stats(post_eps, mean, inv);
+#pragma unroll
+      for (int k = 0; k < ITEMS; ++k) {
+        const int i = 4 * (tid + k * THREADS);
+        if (i < hidden) {
+          const float4 pg = Vec4<TG>::load(post_gain + i);
+          float4 y = {(v[k].x - mean) * inv * pg.x, (v[k].y - mean) * inv * pg.y, (v[k].z - mean) * inv * pg.z,
+                      (v[k].w - mean) * inv * pg.w};
+          if (post_scale) {
+            const float4 ps = Vec4<TG>::load(post_scale + i);
+            y = float4{y.x * ps.x, y.y * ps.y, y.z * ps.z, y.w * ps.w};
+          }
+          v[k] = y;
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+      const int i = 4 * (tid + k * THREADS);
+      if (i < hidden) {
+        v[k] = add4(v[k], Vec4<float>::load(resid + row + i));
+        if (!rows) Vec4<float>::store(resid + row + i, v[k]);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+      const int i = 4 * (tid + k * THREADS);
+      v[k] = i < hidden ? Vec4<float>::load(resid + row + i) : float4{0.f, 0.f, 0.f, 0.f};
+    }
+  }
+  float mean, inv;
+  stats(eps, mean, inv);
+  const size_t orow = static_cast<size_t>(r_out) * hidden;
+#pragma unroll
+  for (int k = 0; k < ITEMS; ++k) {
+    const int i = 4 * (tid + k * THREADS);
+    if (i < hidden) {
+      const float4 gn = Vec4<TG>::load(gain + i);
+      Vec4<TO>::store(out + orow + i, float4{(v[k].x - mean) * inv * gn.x, (v[k].y - mean) * inv * gn.y,
+                                             (v[k].z - mean) * inv * gn.z, (v[k].w - mean) * inv * gn.w});
+    }
+  }
+}
+
 // act[n, i] = g * sigmoid(slope * g) * (u + 1), g = min(gate[n, i], limit), u = clamp(up[n, i], -limit, limit);
 // gate = gu[:, :I], up = gu[:, I:], the partial sums added first. limit <= 0: no clipping.
 __global__ void clipped_glu_kernel(const void* __restrict__ gu, int gu_dt, int n_partials, size_t partial_stride,
@@ -162,6 +243,30 @@ extern "C" int pyre_add_layernorm(float* resid, const void* delta, int delta_dt,
   PYRE_REQUIRE(n >= 0 && hidden > 0 && eps > 0.f, "add_layernorm: bad sizes n=%d hidden=%d", n, hidden);
   PYRE_REQUIRE(hidden <= 64 * kThreads, "add_layernorm: rows of %d elements are more than %d", hidden, 64 * kThreads);
   if (n == 0) return 0;
+  const bool same_gains = (!post_gain || post_gain_dt == gain_dt) && (!post_scale || post_scale_dt == gain_dt);
+  if (!bias && same_gains && hidden % 4 == 0 && hidden <= 4 * 256 * 16 && (!delta || partial_stride % 4 == 0) &&
+      reinterpret_cast<uintptr_t>(delta) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(gain) % 16 == 0 && reinterpret_cast<uintptr_t>(post_gain) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(post_scale) % 16 == 0) {
+    // which shape runs depends on the number of rows; what it computes does not: a row's sums are block
+    // sums of per-thread sums either way, and the two shapes differ in how the elements are dealt to threads
+    const int quads = hidden / 4;
+    const bool few = n <= 128 && quads > 256;  // a decode step: spread each row over more threads
+#define PYRE_LNV(THREADS, ITEMS)                                                                                       \
+  hipLaunchKernelGGL((add_layernorm_vec_kernel<TD, TG, TO, THREADS, ITEMS>), dim3(n), dim3(THREADS), 0, stream, resid, \
+                     static_cast<const TD*>(delta), n_partials, static_cast<size_t>(partial_stride),                   \
+                     static_cast<const TG*>(post_gain), static_cast<const TG*>(post_scale), post_eps,                  \
+                     static_cast<const TG*>(gain), static_cast<TO*>(out), rows, hidden, eps)
+    PYRE_DISPATCH(delta ? delta_dt : kF32, TD, PYRE_DISPATCH(gain_dt, TG, PYRE_DISPATCH(out_dt, TO, {
+      if (few && quads <= 1024) PYRE_LNV(1024, 1);
+      else if (few) PYRE_LNV(1024, 4);
+      else if (quads <= 256) PYRE_LNV(256, 1);
+      else if (quads <= 1024) PYRE_LNV(256, 4);
+      else PYRE_LNV(256, 16);
+    })));
+#undef PYRE_LNV
+    return check_launch("add_layernorm");
+  }
 #define PYRE_LN(ITEMS)                                                                                              \
   hipLaunchKernelGGL(add_layernorm_kernel<ITEMS>, dim3(n), dim3(kThreads), 0, stream, resid, delta, delta_dt,       \
                      n_partials, static_cast<size_t>(partial_stride), bias, bias_dt, post_gain, post_gain_dt,       \

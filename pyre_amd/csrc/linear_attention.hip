@@ -15,6 +15,7 @@
 // Decays, their logarithms, the state and the unit norm are float32 whatever the model's type.
 #include "pyre_api.h"
 #include "pyre_common.h"
+#include "pyre_vec4.h"
 
 using namespace pyre;
 
@@ -47,6 +48,36 @@ __global__ __launch_bounds__(kThreads) void gla_prepare_kernel(
     for (int r = 0; r < rank; ++r) z = fmaf(load_as_float(a2, a2_dt, static_cast<size_t>(c) * rank + r), a1s[r], z);
     if (a2_bias) z += load_as_float(a2_bias, bias_dt, c);
     // log(sigmoid(z)) without overflow on either side
+    const float ls = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
+    xr[2 * hk + c] = ls * inv_tau;
+  }
+}
+
+// The same with four columns to a load and an element's partial sums asked for together (all widths,
+// the first column and the partial sums' stride are multiples of four).
+template <typename TP>
+__global__ __launch_bounds__(kThreads) void gla_prepare_vec_kernel(
+    const TP* __restrict__ proj, int n_partials, size_t partial_stride, int ld, int col0, const void* __restrict__ a2,
+    int a2_dt, const void* __restrict__ a2_bias, int bias_dt, float inv_tau, float* __restrict__ x, int heads, int dk,
+    int dv, int rank) {
+  __shared__ float a1s[kMaxRank];
+  const int n = blockIdx.x, tid = threadIdx.x;
+  const TP* in = proj + static_cast<size_t>(n) * ld + col0;
+  const int hk = heads * dk, hv = heads * dv, width = 3 * hk + 2 * hv;
+  float* xr = x + static_cast<size_t>(n) * width;
+  for (int r = tid; r < rank; r += kThreads) {
+    float v = 0.f;
+    for (int p = 0; p < n_partials; ++p) v += to_float(in[p * partial_stride + 2 * hk + 2 * hv + r]);
+    a1s[r] = v;
+  }
+  for (int i = 4 * tid; i < 2 * hk; i += 4 * kThreads) Vec4<float>::store(xr + i, sum_partials4(in + i, partial_stride, n_partials));
+  for (int i = 4 * tid; i < 2 * hv; i += 4 * kThreads)
+    Vec4<float>::store(xr + 3 * hk + i, sum_partials4(in + 2 * hk + i, partial_stride, n_partials));
+  __syncthreads();
+  for (int c = tid; c < hk; c += kThreads) {
+    float z = 0.f;
+    for (int r = 0; r < rank; ++r) z = fmaf(load_as_float(a2, a2_dt, static_cast<size_t>(c) * rank + r), a1s[r], z);
+    if (a2_bias) z += load_as_float(a2_bias, bias_dt, c);
     const float ls = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
     xr[2 * hk + c] = ls * inv_tau;
   }
@@ -308,6 +339,15 @@ extern "C" int pyre_gla_prepare(const void* proj, int proj_dt, int n_partials, l
   PYRE_REQUIRE(heads > 0 && dk > 0 && dv > 0 && rank > 0 && rank <= kMaxRank, "gla_prepare: bad sizes (rank %d of at most %d)", rank, kMaxRank);
   PYRE_REQUIRE(tau > 0.f, "gla_prepare: tau must be positive");
   if (n <= 0) return 0;
+  const int hk = heads * dk, hv = heads * dv;
+  if (hk % 4 == 0 && hv % 4 == 0 && ld % 4 == 0 && col0 % 4 == 0 && partial_stride % 4 == 0 &&
+      reinterpret_cast<uintptr_t>(proj) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+    PYRE_DISPATCH(proj_dt, TP,
+        hipLaunchKernelGGL(gla_prepare_vec_kernel<TP>, dim3(n), dim3(kThreads), 0, stream, static_cast<const TP*>(proj),
+                           n_partials, static_cast<size_t>(partial_stride), ld, col0, a2, a2_dt, a2_bias, bias_dt,
+                           1.f / tau, x, heads, dk, dv, rank));
+    return check_launch("gla_prepare");
+  }
   hipLaunchKernelGGL(gla_prepare_kernel, dim3(n), dim3(kThreads), 0, stream, proj, proj_dt, n_partials,
                      static_cast<size_t>(partial_stride), ld, col0, a2, a2_dt, a2_bias, bias_dt, 1.f / tau, x, heads, dk,
                      dv, rank);
