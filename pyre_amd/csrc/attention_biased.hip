@@ -275,7 +275,7 @@ __global__ __launch_bounds__(kThreads) void attn_biased_single_kernel(
     int out_ld, const float* __restrict__ gate, float out_scale, const int* __restrict__ tokens,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale, float cap,
-    const float* __restrict__ bias, int far, int window, int keep_first) {
+    const float* __restrict__ bias, int far, int window, int keep_first, float* __restrict__ part) {
   __shared__ __attribute__((aligned(16))) float qs[kMaxHead];
   __shared__ float sc[kSpan];
   __shared__ int row_s[kSpan];
@@ -288,6 +288,10 @@ __global__ __launch_bounds__(kThreads) void attn_biased_single_kernel(
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int kept_end = window > 0 ? min(keep_first, lo) : 0;  // keys 0 .. kept_end - 1, then lo .. pos
   const float* bias_row = bias ? bias + static_cast<size_t>(h) * (far + 1) : nullptr;
+  const int spans_first = (kept_end + kSpan - 1) / kSpan, spans_all = spans_first + (pos - lo) / kSpan + 1;
+  // with scratch for partial results a block takes one span (grid.z of them), else all of them in turn
+  const int span_lo = part ? static_cast<int>(blockIdx.z) : 0, span_hi = part ? min(span_lo + 1, spans_all) : spans_all;
+  if (span_lo >= span_hi) return;
   for (int d = tid; d < dk; d += kThreads) qs[d] = to_float(q[(static_cast<size_t>(n) * nq + h) * dk + d]);
   __syncthreads();
 
@@ -295,8 +299,7 @@ __global__ __launch_bounds__(kThreads) void attn_biased_single_kernel(
   const int g = tid / dv, d = tid % dv;
   const bool active = g < groups;
   float m = -INFINITY, l = 0.f, acc = 0.f;
-  const int spans_first = (kept_end + kSpan - 1) / kSpan, spans_all = spans_first + (pos - lo) / kSpan + 1;
-  for (int span = 0; span < spans_all; ++span) {
+  for (int span = span_lo; span < span_hi; ++span) {
     const int base = span < spans_first ? span * kSpan : lo + (span - spans_first) * kSpan;
     const int cnt = min(kSpan, (span < spans_first ? kept_end : pos + 1) - base);
     float lmax = -INFINITY;
@@ -360,6 +363,40 @@ __global__ __launch_bounds__(kThreads) void attn_biased_single_kernel(
   if (tid < dv) {
     float total = 0.f;
     for (int gg = 0; gg < groups; ++gg) total += accs[gg * dv + tid];
+    if (part) {  // [token of the list][head][span][dv + 2]: unnormalised output, max, sum
+      float* dst = part + ((static_cast<size_t>(blockIdx.x) * nq + h) * gridDim.z + blockIdx.z) * (dv + 2);
+      dst[tid] = total;
+      if (tid == 0) dst[dv] = m, dst[dv + 1] = l;
+      return;
+    }
+    float f = (l > 0.f ? 1.f / l : 0.f) * out_scale;
+    if (gate) f *= gate[static_cast<size_t>(n) * nq + h];
+    out[static_cast<size_t>(n) * out_ld + h * dv + tid] = from_float<T>(total * f);
+  }
+}
+
+// out = gate * out_scale * sum_s acc_s e^(m_s - M) / sum_s l_s e^(m_s - M) over the token's spans, in their order.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void attn_biased_join_kernel(
+    const float* __restrict__ part, T* __restrict__ out, int out_ld, const float* __restrict__ gate, float out_scale,
+    const int* __restrict__ tokens, const int* __restrict__ positions, int nq, int dv, int window, int keep_first,
+    int max_spans) {
+  const int n = tokens ? tokens[blockIdx.x] : blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int pos = positions[n];
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int kept_end = window > 0 ? min(keep_first, lo) : 0;
+  const int spans = min(max_spans, (kept_end + kSpan - 1) / kSpan + (pos - lo) / kSpan + 1);
+  const float* src = part + (static_cast<size_t>(blockIdx.x) * nq + h) * max_spans * (dv + 2);
+  float M = -INFINITY;
+  for (int s = 0; s < spans; ++s) M = fmaxf(M, src[s * (dv + 2) + dv]);
+  const float m_use = M == -INFINITY ? 0.f : M;
+  if (tid < dv) {
+    float total = 0.f, l = 0.f;
+    for (int s = 0; s < spans; ++s) {
+      const float w = expf(src[s * (dv + 2) + dv] - m_use);
+      total = fmaf(src[s * (dv + 2) + tid], w, total);
+      l = fmaf(src[s * (dv + 2) + dv + 1], w, l);
+    }
     float f = (l > 0.f ? 1.f / l : 0.f) * out_scale;
     if (gate) f *= gate[static_cast<size_t>(n) * nq + h];
     out[static_cast<size_t>(n) * out_ld + h * dv + tid] = from_float<T>(total * f);
@@ -441,26 +478,39 @@ extern "C" int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int d
   return check_launch("attn_biased_tile");
 }
 
+// Spans of 128 keys that a token of such a launch can have: those of the kept first tokens and those
+// of the window (or of all `max_keys` keys that a block table holds).
+extern "C" int pyre_attn_biased_spans(int max_keys, int window, int keep_first) {
+  const int seen = window > 0 ? min(window, max_keys) : max_keys;
+  return (window > 0 ? (min(keep_first, max_keys) + kSpan - 1) / kSpan : 0) + (max(seen, 1) - 1) / kSpan + 1;
+}
+
 extern "C" int pyre_attn_biased_single(const void* q, void* out, int out_ld, int dt, const void* k_cache,
                                        const void* v_cache, const float* gate, float out_scale, const int* tokens,
                                        int n, const int* positions, const int* seq_of_token, const int* block_table,
                                        int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale,
-                                       float cap, const float* bias, int far, int window, int keep_first,
-                                       hipStream_t stream) {
+                                       float cap, const float* bias, int far, int window, int keep_first, float* part,
+                                       int max_spans, hipStream_t stream) {
   if (check_geometry("attn_biased_single", nq, nkv, dk, dv, page_size)) return 1;
   PYRE_REQUIRE(known_dtype(dt) && table_stride > 0 && window >= 0 && keep_first >= 0 && far >= 0, "attn_biased_single: bad arguments");
+  PYRE_REQUIRE(!part || (max_spans >= 1 && max_spans <= 65535), "attn_biased_single: %d spans are not a launch", max_spans);
   if (n <= 0) return 0;
+  const dim3 grid(n, nq, part ? max_spans : 1);
 #define PYRE_SINGLE(VEC)                                                                                                 \
   PYRE_DISPATCH(dt, T,                                                                                                    \
-      hipLaunchKernelGGL((attn_biased_single_kernel<T, VEC>), dim3(n, nq), dim3(kThreads), 0, stream,                     \
+      hipLaunchKernelGGL((attn_biased_single_kernel<T, VEC>), grid, dim3(kThreads), 0, stream,                            \
                          static_cast<const T*>(q), static_cast<const T*>(k_cache), static_cast<const T*>(v_cache),        \
                          static_cast<T*>(out), out_ld, gate, out_scale, tokens, positions, seq_of_token, block_table,     \
-                         table_stride, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first))
+                         table_stride, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first, part))
   if (dk % 8 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0) {
     PYRE_SINGLE(true);
   } else {
     PYRE_SINGLE(false);
   }
 #undef PYRE_SINGLE
+  if (part)
+    PYRE_DISPATCH(dt, T,
+        hipLaunchKernelGGL(attn_biased_join_kernel<T>, dim3(n, nq), dim3(kThreads), 0, stream, part, static_cast<T*>(out),
+                           out_ld, gate, out_scale, tokens, positions, nq, dv, window, keep_first, max_spans));
   return check_launch("attn_biased_single");
 }

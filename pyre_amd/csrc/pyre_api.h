@@ -241,8 +241,12 @@ int pyre_attn_biased_single(const void* q, void* out, int out_ld, int dt, const 
                             const void* v_cache, const float* gate, float out_scale, const int* tokens,
                             int n, const int* positions, const int* seq_of_token, const int* block_table,
                             int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale,
-                            float cap, const float* bias, int far, int window, int keep_first,
-                            hipStream_t stream);
+                            float cap, const float* bias, int far, int window, int keep_first, float* part,
+                            int max_spans, hipStream_t stream);
+// part: scratch of n * nq * max_spans * (dv + 2) floats, max_spans = pyre_attn_biased_spans(the most keys a
+// block table holds, window, keep_first): a block then takes one span of 128 keys and a second kernel joins
+// them in their order; null: a block takes all spans of its token and head in turn.
+int pyre_attn_biased_spans(int max_keys, int window, int keep_first);
 
 // ---- gated linear attention (linear_attention.hip) ----
 // proj columns from col0 on: q, k (heads dk each), v, g (heads dv each), the low-rank input (rank).

@@ -11,7 +11,7 @@ from ctypes import c_float, c_int, c_long, c_void_p
 
 from pyre_amd.hip import build as _build
 
-ABI_VERSION = 23
+ABI_VERSION = 24
 
 
 class KernelError(RuntimeError):
@@ -58,7 +58,8 @@ _SIGNATURES = {
     "pyre_scale": [P, L, F, P],
     "pyre_unit_qkv_write": [P, I, I, L, I, I, P, I, P, P, I, P, P, I, I, I, I, I, I, I, F, I, P],
     "pyre_attn_biased_tile": [P, P, I, I, P, P, P, F, P, I, P, P, P, I, I, I, I, I, I, F, F, P, I, I, I, P],
-    "pyre_attn_biased_single": [P, P, I, I, P, P, P, F, P, I, P, P, P, I, I, I, I, I, I, F, F, P, I, I, I, P],
+    "pyre_attn_biased_single": [P, P, I, I, P, P, P, F, P, I, P, P, P, I, I, I, I, I, I, F, F, P, I, I, I, P, I, P],
+    "pyre_attn_biased_spans": [I, I, I],
     "pyre_gla_prepare": [P, I, I, L, I, I, P, I, P, I, F, P, I, I, I, I, I, P],
     "pyre_gla_scan": [P, P, P, P, P, I, I, I, I, F, P],
     "pyre_gla_chunks": [P, P, P, P, P, P, I, I, I, I, I, I, F, P],

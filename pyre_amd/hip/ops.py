@@ -288,17 +288,33 @@ def attn_biased_tile(q, out, k_cache, v_cache, gate, out_scale, tiles, n_tiles, 
          float(scale), float(cap), _ptr(bias), int(far), int(window), int(keep_first), _stream())
 
 
+def attn_biased_spans(table_width: int, page_size: int, window: int, keep_first: int) -> int:
+    """Spans of 128 keys that a token can have when its block table is ``table_width`` pages wide."""
+    from pyre_amd.hip.lib import lib
+
+    return int(lib().pyre_attn_biased_spans(max(1, table_width * page_size), int(window), int(keep_first)))
+
+
 def attn_biased_single(q, out, k_cache, v_cache, gate, out_scale, tokens, n, positions, seq_of_token,
-                       block_table, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first) -> None:
-    """The same for ``n`` tokens one by one (``tokens``: which of the flat batch, None: the first n)."""
+                       block_table, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first,
+                       scratch: torch.Tensor | None = None) -> None:
+    """The same for ``n`` tokens one by one (``tokens``: which of the flat batch, None: the first n). ``scratch``
+    (float32, ``n * nq * attn_biased_spans(...) * (dv + 2)`` elements): a block per span of 128 keys and a second
+    kernel that joins them, instead of a block per token and head that takes its spans in turn."""
     _attn_biased_common(q, out, k_cache, v_cache, gate, positions, seq_of_token, block_table, bias, far,
                         nq, nkv, dk, dv, page_size)
     if tokens is not None:
         _dev(tokens), _i32("tokens", tokens, n)
+    spans = 0
+    if scratch is not None:
+        _dev(scratch)
+        spans = attn_biased_spans(block_table.shape[1], page_size, window, keep_first)
+        if scratch.dtype != torch.float32 or not scratch.is_contiguous() or scratch.numel() < n * nq * spans * (dv + 2):
+            raise KernelError(f"attn_biased_single: scratch of {n * nq * spans * (dv + 2)} float32 elements needed")
     call("pyre_attn_biased_single", q.data_ptr(), out.data_ptr(), out.stride(0), dtype_code(q), k_cache.data_ptr(),
          v_cache.data_ptr(), _ptr(gate), float(out_scale), _ptr(tokens), n, positions.data_ptr(),
          seq_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0), nq, nkv, dk, dv, page_size,
-         float(scale), float(cap), _ptr(bias), int(far), int(window), int(keep_first), _stream())
+         float(scale), float(cap), _ptr(bias), int(far), int(window), int(keep_first), _ptr(scratch), spans, _stream())
 
 
 GLA_MAX_RANK = 512     #: the widest low-rank input of the decay (linear_attention.hip)

@@ -11,6 +11,10 @@ from pyre_amd.parts.base import Mixer, ParallelMixerSpec, TensorSpec, make_part,
 from pyre_amd.parts.linear import Linear
 
 
+#: columns of a shared input product at which a branch's own begin
+COLUMN_ALIGN = 8
+
+
 class BranchMixer(Mixer):
     """A mixer of the form out(f(in_1 h, in_2 h, ...)): all its input matrices multiply the rows it is
     given, and one output matrix multiplies what it makes of them. It says which matrices these are
@@ -102,14 +106,24 @@ class ParallelMixer(Mixer):
         return [s for b in self.branches for s in (*b.in_tensors(), b.out_tensor(), *b.other_tensors())]
 
     def bind(self, tensors, runtime) -> None:
-        col = 0
+        # every branch's columns start at a multiple of eight (rows of zeros between them), so that the
+        # kernels which finish the product read them in 16-byte pieces
+        col, parts = 0, []
         self.first_column = []
         for b in self.branches:
             self.first_column.append(col)
-            col += sum(tensors[s.name].shape[0] for s in b.in_tensors())
+            mine = [take(tensors, s.name) for s in b.in_tensors()]
+            rows = sum(t.shape[0] for t in mine)
+            pad = -rows % COLUMN_ALIGN
+            if pad and b is not self.branches[-1]:
+                mine.append(torch.zeros(pad, mine[0].shape[1], dtype=mine[0].dtype, device=mine[0].device))
+                rows += pad
+            parts += mine
+            col += rows
         self.proj = Linear(self.spec.hidden_size, col, "mix.in")
         self.out = Linear(self.inner, self.spec.hidden_size, "mix.out")
-        self.proj.set(_stacked([s.name for b in self.branches for s in b.in_tensors()], tensors, 0))
+        self.proj.set(torch.cat(parts, dim=0))
+        del parts, mine
         self.out.set(_stacked([b.out_tensor().name for b in self.branches], tensors, 1))
         for b in self.branches:
             b.bind_others(tensors, runtime)

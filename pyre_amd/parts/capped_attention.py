@@ -113,5 +113,10 @@ class CappedAttention(BranchMixer):
             ops.attn_biased_tile(q, o, k_pages, v_pages, gate, scale, ctx.arrays["attention.prefill_tiles"], len(tiles),
                                  ctx.positions, ctx.seq_of_token, cache.table, *shape)
         if len(singles):
+            # a block per span of 128 keys, joined by a second kernel: a step of few tokens fills the chip that way
+            spans = ops.attn_biased_spans(cache.table.shape[1], cache.page_size, s.window, s.keep_first)
+            scratch = None
+            if spans > 1:
+                scratch = ws.get("cattn.spans", (len(singles) * s.num_heads * spans * (s.value_dim + 2),), torch.float32)
             ops.attn_biased_single(q, o, k_pages, v_pages, gate, scale, ctx.arrays["attention.decode_tokens"],
-                                   len(singles), ctx.positions, ctx.seq_of_token, cache.table, *shape)
+                                   len(singles), ctx.positions, ctx.seq_of_token, cache.table, *shape, scratch=scratch)
