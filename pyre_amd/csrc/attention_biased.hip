@@ -84,6 +84,8 @@ __global__ __launch_bounds__(kThreads) void unit_qkv_write_kernel(
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 constexpr int kKeys = 32;
 constexpr int kTileMaxKeyHead = 128;  // the queries of a block's four heads lie in LDS
+constexpr int kVtLd = kKeys + 4;      // a row of transposed values: 16-byte reads of four keys
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // Eight consecutive elements as floats in one or two 16-byte loads; p is aligned to 16 bytes.
 __device__ inline void load8(const float* p, float (&v)[8]) {
@@ -100,9 +102,17 @@ __device__ inline void load8(const bf16* p, float (&v)[8]) {
   }
 }
 
+// tanh(x) = sign(x) (1 - e) / (1 + e) with e = exp(-2 |x|) <= 1: one exponential and one division, no
+// branches; its absolute error is a few 1e-8 everywhere (the library's branches cost a tile of scores
+// more than both of its matrix products).
+__device__ inline float tanh_by_exp(float x) {
+  const float e = expf(-2.f * fabsf(x));
+  return copysignf((1.f - e) / (1.f + e), x);
+}
+
 __device__ inline float shaped_score(float raw, float scale, float cap, const float* bias_row, int dist, int far) {
   float s = raw * scale;
-  if (cap > 0.f) s = cap * tanhf(s / cap);
+  if (cap > 0.f) s = cap * tanh_by_exp(s / cap);
   if (bias_row) s += bias_row[min(dist, far)];
   return s;
 }
@@ -120,11 +130,13 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, int nq, int nkv, int dk, int dkp, int dv, int page_size, float scale, float cap,
     const float* __restrict__ bias, int far, int window, int keep_first) {
-  extern __shared__ float lds[];
-  float* Ks = lds;                              // [kKeys][dkp + 1]
-  float* Qs = Ks + kKeys * (dkp + 1);           // [4 waves][32 tokens][dkp + 1]
-  float* Vt = Qs + 4 * 32 * (dkp + 1);          // [32 NV][kKeys + 1]
-  __shared__ int page_s[kKeys];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  // rows of keys and queries hold the even elements first, then the odd ones: a lane's operands of four
+  // steps of the first product are then one 16-byte read
+  float* Ks = lds;                              // [kKeys][dkp + 4]
+  float* Qs = Ks + kKeys * (dkp + 4);           // [4 waves][32 tokens][dkp + 4]
+  float* Vt = Qs + 4 * 32 * (dkp + 4);          // [32 NV][kVtLd]
+  __shared__ int page_s[2][kKeys];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, h = lane >> 5, c = lane & 31;
   const int n_rep = nq / nkv, hgroups = (n_rep + 3) / 4;
   const int kvh = blockIdx.y / hgroups, hin = (blockIdx.y % hgroups) * 4 + wave;
@@ -134,7 +146,7 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
   if (ntok <= 0) return;
   const int pos0 = positions[t0];
   const int* table = block_table + static_cast<size_t>(seq_of_token[t0]) * table_stride;
-  const int ldk = dkp + 1;
+  const int ldk = dkp + 4, half = dkp / 2;
 
   const bool live = active && c < ntok;
   const int hi = c < ntok ? pos0 + c : pos0;
@@ -143,12 +155,22 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
   const float* bias_row = bias ? bias + static_cast<size_t>(head) * (far + 1) : nullptr;
   {  // this wave's queries: Qs[wave][token][d], zeros where there is no token or no element
     float* mine = Qs + wave * 32 * ldk;
-    for (int i = lane; i < 32 * dkp; i += 64) {
-      const int t = i / dkp, d = i % dkp;
-      mine[t * ldk + d] = active && t < ntok && d < dk ? to_float(q[(static_cast<size_t>(t0 + t) * nq + head) * dk + d]) : 0.f;
+    if (VEC) {
+      for (int i = lane; i < 32 * (dkp / 8); i += 64) {
+        const int t = i / (dkp / 8), d = 8 * (i % (dkp / 8));
+        float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (active && t < ntok && d < dk) load8(q + (static_cast<size_t>(t0 + t) * nq + head) * dk + d, v);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) mine[t * ldk + (u & 1) * half + ((d + u) >> 1)] = v[u];
+      }
+    } else {
+      for (int i = lane; i < 32 * dkp; i += 64) {
+        const int t = i / dkp, d = i % dkp;
+        mine[t * ldk + (d & 1) * half + (d >> 1)] = active && t < ntok && d < dk ? to_float(q[(static_cast<size_t>(t0 + t) * nq + head) * dk + d]) : 0.f;
+      }
     }
   }
-  const float* myq = Qs + wave * 32 * ldk + c * ldk;
+  const float* myq = Qs + wave * 32 * ldk + c * ldk + h * half;
   f32x16 o[NV];
 #pragma unroll
   for (int dt = 0; dt < NV; ++dt)
@@ -163,66 +185,107 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
   const int n_first = kept_end > 0 ? (kept_end - 1) / kKeys + 1 : 0;
   const int chunk_b = max(lo_all / kKeys, n_first);
   const int n_chunks = n_first + (hi_all / kKeys - chunk_b + 1);
-  for (int it = 0; it < n_chunks; ++it) {
-    const int chunk = it < n_first ? it : chunk_b + (it - n_first);
-    const int key0 = chunk * kKeys;
-    __syncthreads();  // the previous chunk has been read by every wave (and the queries are written)
-    if (tid < kKeys) {
-      const int key = key0 + tid, entry = key / page_size;
-      page_s[tid] = key <= hi_all && entry < table_stride ? table[entry] : -1;
+  // VEC: the next chunk's keys and values are asked for (into registers) before the current chunk is
+  // multiplied, and go to LDS when every wave is done with it
+  constexpr int KI = kKeys * (kTileMaxKeyHead / 8) / kThreads, VI = (kKeys * 4 * NV + kThreads - 1) / kThreads;
+  float kreg[KI][8], vreg[VI][8];
+  auto chunk_key0 = [&](int it) { return (it < n_first ? it : chunk_b + (it - n_first)) * kKeys; };
+  auto page_of = [&](int key) {
+    const int entry = key / page_size;
+    return key <= hi_all && entry < table_stride ? table[entry] : -1;
+  };
+  auto ask = [&](int it) {
+    const int key0 = chunk_key0(it), kg = dkp / 8;
+    if (tid < kKeys) page_s[it & 1][tid] = page_of(key0 + tid);
+#pragma unroll
+    for (int k = 0; k < KI; ++k) {
+      const int i = tid + k * kThreads, key = key0 + i / kg, d = 8 * (i % kg);
+      const int page = i < kKeys * kg ? page_of(key) : -1;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) kreg[k][u] = 0.f;
+      if (page >= 0 && d < dk) load8(k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + key % page_size) * dk + d, kreg[k]);
     }
-    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < VI; ++k) {
+      const int i = tid + k * kThreads, key = key0 + i / (4 * NV), d = 8 * (i % (4 * NV));
+      const int page = i < kKeys * 4 * NV ? page_of(key) : -1;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) vreg[k][u] = 0.f;
+      if (page >= 0 && d < dv) load8(v_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + key % page_size) * dv + d, vreg[k]);
+    }
+  };
+  auto stash = [&]() {
+    const int kg = dkp / 8;
+#pragma unroll
+    for (int k = 0; k < KI; ++k) {
+      const int i = tid + k * kThreads, key = i / kg, d = 8 * (i % kg);
+      if (i < kKeys * kg)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) Ks[key * ldk + (u & 1) * half + ((d + u) >> 1)] = kreg[k][u];
+    }
+#pragma unroll
+    for (int k = 0; k < VI; ++k) {
+      const int i = tid + k * kThreads, key = i / (4 * NV), d = 8 * (i % (4 * NV));
+      if (i < kKeys * 4 * NV)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) Vt[(d + u) * kVtLd + key] = vreg[k][u];
+    }
+  };
+  if (VEC) ask(0);
+  for (int it = 0; it < n_chunks; ++it) {
+    const int key0 = chunk_key0(it);
+    const int* pages = page_s[it & 1];
+    __syncthreads();  // the previous chunk has been read by every wave (and the queries are written)
     if (VEC) {
-      const int kg = dkp / 8;
-      for (int i = tid; i < kKeys * kg; i += kThreads) {
-        const int key = i / kg, d = 8 * (i % kg), page = page_s[key];
-        float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        if (page >= 0 && d < dk)
-          load8(k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + (key0 + key) % page_size) * dk + d, v);
-#pragma unroll
-        for (int u = 0; u < 8; ++u) Ks[key * ldk + d + u] = v[u];
-      }
-      for (int i = tid; i < kKeys * 4 * NV; i += kThreads) {
-        const int key = i / (4 * NV), d = 8 * (i % (4 * NV)), page = page_s[key];
-        float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        if (page >= 0 && d < dv)
-          load8(v_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + (key0 + key) % page_size) * dv + d, v);
-#pragma unroll
-        for (int u = 0; u < 8; ++u) Vt[(d + u) * (kKeys + 1) + key] = v[u];
-      }
+      stash();
     } else {
+      if (tid < kKeys) page_s[it & 1][tid] = page_of(key0 + tid);
+      __syncthreads();
       for (int i = tid; i < kKeys * dkp; i += kThreads) {
-        const int key = i / dkp, d = i % dkp, page = page_s[key];
+        const int key = i / dkp, d = i % dkp, page = pages[key];
         float v = 0.f;
         if (page >= 0 && d < dk)
           v = to_float(k_cache[((static_cast<size_t>(page) * nkv + kvh) * page_size + (key0 + key) % page_size) * dk + d]);
-        Ks[key * ldk + d] = v;
+        Ks[key * ldk + (d & 1) * half + (d >> 1)] = v;
       }
       for (int i = tid; i < kKeys * 32 * NV; i += kThreads) {
-        const int key = i / (32 * NV), d = i % (32 * NV), page = page_s[key];
+        const int key = i / (32 * NV), d = i % (32 * NV), page = pages[key];
         float v = 0.f;
         if (page >= 0 && d < dv)
           v = to_float(v_cache[((static_cast<size_t>(page) * nkv + kvh) * page_size + (key0 + key) % page_size) * dv + d]);
-        Vt[d * (kKeys + 1) + key] = v;
+        Vt[d * kVtLd + key] = v;
       }
     }
     __syncthreads();
+    if (VEC && it + 1 < n_chunks) ask(it + 1);
     if (!active) continue;
 
     f32x16 s;
 #pragma unroll
     for (int i = 0; i < 16; ++i) s[i] = 0.f;
-    const float* krow = Ks + c * ldk;
-    for (int st = 0; st < dkp / 2; ++st)
-      s = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[2 * st + h], myq[2 * st + h], s, 0, 0, 0);
+    const float* krow = Ks + c * ldk + h * half;
+#pragma unroll 4
+    for (int st = 0; st < half; st += 4) {  // elements 2 st + h, ..., 2 (st + 3) + h of the key and the query
+      const f32x4 k4 = *reinterpret_cast<const f32x4*>(krow + st), q4 = *reinterpret_cast<const f32x4*>(myq + st);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) s = __builtin_amdgcn_mfma_f32_32x32x2f32(k4[u], q4[u], s, 0, 0, 0);
+    }
 
     // element i of s: key key0 + 8 (i / 4) + 4 h + i % 4, token c
+    // the biases of the lane's sixteen distances, asked for together (a key that is not seen reads a distance that is there)
+    float bv[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int key = key0 + 8 * (i >> 2) + 4 * h + (i & 3);
+      bv[i] = bias_row ? bias_row[min(max(hi - key, 0), far)] : 0.f;
+    }
     float mx = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int kk = 8 * (i >> 2) + 4 * h + (i & 3), key = key0 + kk;
-      const bool seen = key <= hi && (key >= lo || key < keep) && page_s[kk] >= 0;
-      s[i] = seen ? shaped_score(s[i], scale, cap, bias_row, hi - key, far) : -INFINITY;
+      const bool seen = key <= hi && (key >= lo || key < keep) && pages[kk] >= 0;
+      const float shaped = shaped_score(s[i], scale, cap, nullptr, 0, 0) + bv[i];
+      s[i] = seen ? shaped : -INFINITY;
       mx = fmaxf(mx, s[i]);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
@@ -244,9 +307,11 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
 #pragma unroll
     for (int dt = 0; dt < NV; ++dt)
 #pragma unroll
-      for (int st = 0; st < 16; ++st)
-        o[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(Vt[(32 * dt + c) * (kKeys + 1) + 8 * (st >> 2) + 4 * h + (st & 3)],
-                                                     s[st], o[dt], 0, 0, 0);
+      for (int a = 0; a < 4; ++a) {
+        const f32x4 v4 = *reinterpret_cast<const f32x4*>(&Vt[(32 * dt + c) * kVtLd + 8 * a + 4 * h]);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) o[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(v4[u], s[4 * a + u], o[dt], 0, 0, 0);
+      }
   }
 
   if (!active) return;
@@ -443,7 +508,7 @@ extern "C" int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int d
   PYRE_REQUIRE(nkv * hgroups <= 65535, "attn_biased_tile: grid too large");
   const int dkp = (dk + 31) / 32 * 32, nv = (dv + 31) / 32;
   const int nvp = nv <= 1 ? 1 : nv <= 2 ? 2 : nv <= 4 ? 4 : 8;
-  const size_t lds = sizeof(float) * (static_cast<size_t>(kKeys + 4 * 32) * (dkp + 1) + 32 * nvp * (kKeys + 1));
+  const size_t lds = sizeof(float) * (static_cast<size_t>(kKeys + 4 * 32) * (dkp + 4) + 32 * nvp * kVtLd);
   const dim3 grid(n_tiles, nkv * hgroups);
 #define PYRE_TILE(T, NV, VEC)                                                                                           \
   do {                                                                                                               \
@@ -467,7 +532,7 @@ extern "C" int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int d
     default: PYRE_TILE(T, 8, VEC); break;   \
   }
   const bool vec = dk % 8 == 0 && dv % 8 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 &&
-                   reinterpret_cast<uintptr_t>(v_cache) % 16 == 0;
+                   reinterpret_cast<uintptr_t>(v_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0;
   if (dt == kF32) {
     if (vec) { PYRE_TILE_NV(float, true) } else { PYRE_TILE_NV(float, false) }
   } else {
