@@ -266,7 +266,8 @@ def designs(args) -> dict:
         times = [prefill_once() for _ in range(4)][1:]
         ms = statistics.median(times) * 1e3
         res["prefill"] = {"tokens": PREFILL_TOKENS, "ms": round(ms, 3), "tok_s": round(PREFILL_TOKENS / ms * 1e3, 1)}
-        res["prefill_kernels_us"] = kernels_of(prefill_once, 1)
+        if not args.no_breakdown:
+            res["prefill_kernels_us"] = kernels_of(prefill_once, 1)
         for batch in batches:
             sched = Scheduler(engine, max_batch=batch)
             steps = args.steps
@@ -287,7 +288,7 @@ def designs(args) -> dict:
                 blocks.append(time.perf_counter() - t)
             dt = sorted(blocks)[1]
             res[f"decode_b{batch}"] = {"ms": round(dt / steps * 1e3, 4), "tok_s": round(batch * steps / dt, 1)}
-            if batch == batches[0]:
+            if batch == batches[0] and not args.no_breakdown:
                 res["decode_kernels_us"] = kernels_of(lambda: [sched.step() for _ in range(4)], 4)
             for r in list(sched.running):
                 engine.finish(r.seq_id)

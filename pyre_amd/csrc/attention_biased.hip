@@ -23,6 +23,7 @@
 // every sum of a token depends on its own bounds alone.
 #include "pyre_api.h"
 #include "pyre_common.h"
+#include "pyre_vec4.h"
 
 using namespace pyre;
 
@@ -80,6 +81,43 @@ __global__ __launch_bounds__(kThreads) void unit_qkv_write_kernel(
     for (int h = tid; h < nq; h += kThreads) gate_out[static_cast<size_t>(n) * nq + h] = 1.f / (1.f + expf(-value(v0 + nkv * dv + h)));
 }
 
+// The same with four elements to a load and an element's partial sums asked for together (head sizes,
+// the product's width, first column and stride are multiples of four; queries stored as the cache's type).
+template <typename TP, typename TC>
+__global__ __launch_bounds__(kThreads) void unit_qkv_write_vec_kernel(
+    const TP* __restrict__ proj, int n_partials, size_t partial_stride, int ld, int col0, TC* __restrict__ q_out,
+    TC* __restrict__ k_cache, TC* __restrict__ v_cache, float* __restrict__ gate_out, const int* __restrict__ slots,
+    int nq, int nkv, int dk, int dv, int page_size, int unit_norm, float eps, int gated, int write_kv) {
+  const int n = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const TP* in = proj + static_cast<size_t>(n) * ld + col0;
+  const int slot = write_kv ? slots[n] : -1;
+  const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+  for (int head = wave; head < nq + nkv; head += kThreads / kWave) {  // a wave a head, four elements a lane
+    const int e = 4 * lane;
+    float4 x = {0.f, 0.f, 0.f, 0.f};
+    if (e < dk) x = sum_partials4(in + head * dk + e, partial_stride, n_partials);
+    float inv = 1.f;
+    if (unit_norm) inv = 1.f / sqrtf(wave_sum((x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w)) / static_cast<float>(dk) + eps);
+    if (e >= dk) continue;
+    const float4 y = {x.x * inv, x.y * inv, x.z * inv, x.w * inv};
+    if (head < nq) Vec4<TC>::store(q_out + (static_cast<size_t>(n) * nq + head) * dk + e, y);
+    else if (slot >= 0) Vec4<TC>::store(k_cache + ((static_cast<size_t>(page) * nkv + (head - nq)) * page_size + off) * dk + e, y);
+  }
+  const int v0 = (nq + nkv) * dk;
+  if (slot >= 0)
+    for (int i = 4 * tid; i < nkv * dv; i += 4 * kThreads) {
+      const int g = i / dv, e = i % dv;
+      Vec4<TC>::store(v_cache + ((static_cast<size_t>(page) * nkv + g) * page_size + off) * dv + e,
+                      sum_partials4(in + v0 + i, partial_stride, n_partials));
+    }
+  if (gated)
+    for (int h = tid; h < nq; h += kThreads) {
+      float v = 0.f;
+      for (int p = 0; p < n_partials; ++p) v += to_float(in[p * partial_stride + v0 + nkv * dv + h]);
+      gate_out[static_cast<size_t>(n) * nq + h] = 1.f / (1.f + expf(-v));
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 constexpr int kKeys = 32;
@@ -129,13 +167,15 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
     int out_ld, const float* __restrict__ gate, float out_scale, const int* __restrict__ tiles,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, int nq, int nkv, int dk, int dkp, int dv, int page_size, float scale, float cap,
-    const float* __restrict__ bias, int far, int window, int keep_first) {
+    const float* __restrict__ bias, int far, int window, int keep_first, int tab_lds, int bias_lds) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // rows of keys and queries hold the even elements first, then the odd ones: a lane's operands of four
   // steps of the first product are then one 16-byte read
   float* Ks = lds;                              // [kKeys][dkp + 4]
   float* Qs = Ks + kKeys * (dkp + 4);           // [4 waves][32 tokens][dkp + 4]
   float* Vt = Qs + 4 * 32 * (dkp + 4);          // [32 NV][kVtLd]
+  int* tab_s = reinterpret_cast<int*>(Vt + 32 * NV * kVtLd);  // [tab_lds]: the request's block table, if it fits
+  float* bias_s = reinterpret_cast<float*>(tab_s + tab_lds);  // [4][far + 1]: the four heads' biases, if they fit
   __shared__ int page_s[2][kKeys];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, h = lane >> 5, c = lane & 31;
   const int n_rep = nq / nkv, hgroups = (n_rep + 3) / 4;
@@ -153,6 +193,11 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
   const int lo = window > 0 ? max(0, hi - window + 1) : 0;
   const int keep = window > 0 ? keep_first : 0;
   const float* bias_row = bias ? bias + static_cast<size_t>(head) * (far + 1) : nullptr;
+  for (int i = tid; i < tab_lds; i += kThreads) tab_s[i] = table[i];
+  if (bias && bias_lds) {  // from here on the biases are read from LDS: no load that a wait for them would queue behind
+    for (int i = lane; i <= far; i += 64) bias_s[wave * (far + 1) + i] = bias_row[i];
+    bias_row = bias_s + wave * (far + 1);
+  }
   {  // this wave's queries: Qs[wave][token][d], zeros where there is no token or no element
     float* mine = Qs + wave * 32 * ldk;
     if (VEC) {
@@ -192,7 +237,8 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
   auto chunk_key0 = [&](int it) { return (it < n_first ? it : chunk_b + (it - n_first)) * kKeys; };
   auto page_of = [&](int key) {
     const int entry = key / page_size;
-    return key <= hi_all && entry < table_stride ? table[entry] : -1;
+    if (key > hi_all || entry >= table_stride) return -1;
+    return entry < tab_lds ? tab_s[entry] : table[entry];
   };
   auto ask = [&](int it) {
     const int key0 = chunk_key0(it), kg = dkp / 8;
@@ -231,6 +277,7 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
         for (int u = 0; u < 8; ++u) Vt[(d + u) * kVtLd + key] = vreg[k][u];
     }
   };
+  __syncthreads();  // the table and the biases are in LDS
   if (VEC) ask(0);
   for (int it = 0; it < n_chunks; ++it) {
     const int key0 = chunk_key0(it);
@@ -486,6 +533,16 @@ extern "C" int pyre_unit_qkv_write(const void* proj, int proj_dt, int n_partials
   PYRE_REQUIRE(!write_kv || (k_cache && v_cache && slots), "unit_qkv_write: a cache write needs caches and slots");
   PYRE_REQUIRE(!unit_norm || eps > 0.f, "unit_qkv_write: eps must be positive");
   if (n <= 0) return 0;
+  if (dk % 4 == 0 && dv % 4 == 0 && ld % 4 == 0 && col0 % 4 == 0 && partial_stride % 4 == 0 && q_dt == cache_dt &&
+      reinterpret_cast<uintptr_t>(proj) % 16 == 0 && reinterpret_cast<uintptr_t>(q_out) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0) {
+    PYRE_DISPATCH(proj_dt, TP, PYRE_DISPATCH(cache_dt, TC,
+        hipLaunchKernelGGL((unit_qkv_write_vec_kernel<TP, TC>), dim3(n), dim3(kThreads), 0, stream,
+                           static_cast<const TP*>(proj), n_partials, static_cast<size_t>(partial_stride), ld, col0,
+                           static_cast<TC*>(q_out), static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), gate_out, slots,
+                           nq, nkv, dk, dv, page_size, unit_norm, eps, gate_out ? 1 : 0, write_kv)));
+    return check_launch("unit_qkv_write");
+  }
   PYRE_DISPATCH(cache_dt, TC,
       hipLaunchKernelGGL(unit_qkv_write_kernel<TC>, dim3(n), dim3(kThreads), 0, stream, proj, proj_dt, n_partials,
                          static_cast<size_t>(partial_stride), ld, col0, q_out, q_dt, static_cast<TC*>(k_cache),
@@ -508,7 +565,13 @@ extern "C" int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int d
   PYRE_REQUIRE(nkv * hgroups <= 65535, "attn_biased_tile: grid too large");
   const int dkp = (dk + 31) / 32 * 32, nv = (dv + 31) / 32;
   const int nvp = nv <= 1 ? 1 : nv <= 2 ? 2 : nv <= 4 ? 4 : 8;
-  const size_t lds = sizeof(float) * (static_cast<size_t>(kKeys + 4 * 32) * (dkp + 4) + 32 * nvp * kVtLd);
+  size_t lds = sizeof(float) * (static_cast<size_t>(kKeys + 4 * 32) * (dkp + 4) + 32 * nvp * kVtLd);
+  // what is left of a compute unit's LDS takes the request's block table and the four heads' biases
+  const size_t budget = 158 * 1024;
+  const int tab_lds = lds + sizeof(int) * table_stride <= budget ? table_stride : 0;
+  lds += sizeof(int) * tab_lds;
+  const int bias_lds = bias && lds + sizeof(float) * 4 * (far + 1) <= budget ? 1 : 0;
+  lds += bias_lds ? sizeof(float) * 4 * (far + 1) : 0;
   const dim3 grid(n_tiles, nkv * hgroups);
 #define PYRE_TILE(T, NV, VEC)                                                                                           \
   do {                                                                                                               \
@@ -522,7 +585,7 @@ extern "C" int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int d
     hipLaunchKernelGGL((attn_biased_tile_kernel<T, NV, VEC>), grid, dim3(kThreads), lds, stream, static_cast<const T*>(q), \
                        static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), static_cast<T*>(out), out_ld, \
                        gate, out_scale, tiles, positions, seq_of_token, block_table, table_stride, nq, nkv, dk, dkp,  \
-                       dv, page_size, scale, cap, bias, far, window, keep_first);                                    \
+                       dv, page_size, scale, cap, bias, far, window, keep_first, tab_lds, bias_lds);                 \
   } while (0)
 #define PYRE_TILE_NV(T, VEC)                \
   switch (nvp) {                            \

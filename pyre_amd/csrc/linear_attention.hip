@@ -55,10 +55,10 @@ __global__ __launch_bounds__(kThreads) void gla_prepare_kernel(
 
 // The same with four columns to a load and an element's partial sums asked for together (all widths,
 // the first column and the partial sums' stride are multiples of four).
-template <typename TP>
+template <typename TP, typename TA>
 __global__ __launch_bounds__(kThreads) void gla_prepare_vec_kernel(
-    const TP* __restrict__ proj, int n_partials, size_t partial_stride, int ld, int col0, const void* __restrict__ a2,
-    int a2_dt, const void* __restrict__ a2_bias, int bias_dt, float inv_tau, float* __restrict__ x, int heads, int dk,
+    const TP* __restrict__ proj, int n_partials, size_t partial_stride, int ld, int col0, const TA* __restrict__ a2,
+    const void* __restrict__ a2_bias, int bias_dt, float inv_tau, float* __restrict__ x, int heads, int dk,
     int dv, int rank) {
   __shared__ float a1s[kMaxRank];
   const int n = blockIdx.x, tid = threadIdx.x;
@@ -76,7 +76,9 @@ __global__ __launch_bounds__(kThreads) void gla_prepare_vec_kernel(
   __syncthreads();
   for (int c = tid; c < hk; c += kThreads) {
     float z = 0.f;
-    for (int r = 0; r < rank; ++r) z = fmaf(load_as_float(a2, a2_dt, static_cast<size_t>(c) * rank + r), a1s[r], z);
+    const TA* row = a2 + static_cast<size_t>(c) * rank;
+#pragma unroll 8
+    for (int r = 0; r < rank; ++r) z = fmaf(to_float(row[r]), a1s[r], z);  // typed loads: eight of them on their way together
     if (a2_bias) z += load_as_float(a2_bias, bias_dt, c);
     const float ls = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
     xr[2 * hk + c] = ls * inv_tau;
@@ -342,10 +344,10 @@ extern "C" int pyre_gla_prepare(const void* proj, int proj_dt, int n_partials, l
   const int hk = heads * dk, hv = heads * dv;
   if (hk % 4 == 0 && hv % 4 == 0 && ld % 4 == 0 && col0 % 4 == 0 && partial_stride % 4 == 0 &&
       reinterpret_cast<uintptr_t>(proj) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
-    PYRE_DISPATCH(proj_dt, TP,
-        hipLaunchKernelGGL(gla_prepare_vec_kernel<TP>, dim3(n), dim3(kThreads), 0, stream, static_cast<const TP*>(proj),
-                           n_partials, static_cast<size_t>(partial_stride), ld, col0, a2, a2_dt, a2_bias, bias_dt,
-                           1.f / tau, x, heads, dk, dv, rank));
+    PYRE_DISPATCH(proj_dt, TP, PYRE_DISPATCH(a2_dt, TA,
+        hipLaunchKernelGGL((gla_prepare_vec_kernel<TP, TA>), dim3(n), dim3(kThreads), 0, stream,
+                           static_cast<const TP*>(proj), n_partials, static_cast<size_t>(partial_stride), ld, col0,
+                           static_cast<const TA*>(a2), a2_bias, bias_dt, 1.f / tau, x, heads, dk, dv, rank)));
     return check_launch("gla_prepare");
   }
   hipLaunchKernelGGL(gla_prepare_kernel, dim3(n), dim3(kThreads), 0, stream, proj, proj_dt, n_partials,
