@@ -46,7 +46,8 @@ def build_mafurax(cfg: MafuraxConfig) -> ModelSpec:
     layers = []
     for i, layer in enumerate(cfg.layers):
         p = f"l{i}"
-        ff = {}
+        # a layer without a feed-forward: a file may still hold that half's norms and scale; nothing reads them
+        ff = dict(unused=(f"{p}.norm2", f"{p}.norm2b", f"{p}.ls2"))
         if layer.mlp is not None:
             ff = dict(feed_forward=FEED_FORWARDS[type(layer.mlp)](cfg, layer.mlp, f"{p}.mlp"), feed_forward_norm=norm(f"{p}.norm2"),
                       feed_forward_post_norm=norm(f"{p}.norm2b"), feed_forward_scale=f"{p}.ls2")

@@ -58,6 +58,9 @@ class TensorSpec:
     #: a size that only the file knows is None in ``shape`` (the part reads it off the tensor when it
     #: binds); the random-weights mode then draws this shape
     random_shape: tuple[int, ...] | None = None
+    #: a tensor that a file may hold though nothing reads it (the norm of a sublayer that this layer
+    #: does not have): neither missed when absent nor refused when present, never drawn
+    optional: bool = False
 
     def fits(self, shape) -> bool:
         shape = tuple(shape)
@@ -407,6 +410,8 @@ class SandwichBlockSpec:
     feed_forward_norm: Any = None
     feed_forward_post_norm: Any = None
     feed_forward_scale: str | None = None
+    #: tensors over the hidden size that a file may hold for this layer though nothing reads them
+    unused: tuple = ()
     kind: ClassVar[str] = "sandwich"
 
 

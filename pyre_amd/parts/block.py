@@ -87,13 +87,17 @@ class SandwichBlock(Block):
     def tensor_specs(self) -> list[TensorSpec]:
         hidden = self.mixer_norm.spec.hidden_size
         return [s for p in self.parts() for s in p.tensor_specs()] + \
-               [TensorSpec(n, (hidden,), init="gain") for n in self._scale_names()]
+               [TensorSpec(n, (hidden,), init="gain") for n in self._scale_names()] + \
+               [TensorSpec(n, (hidden,), init="gain", optional=True) for n in self.spec.unused]
 
     def bind(self, tensors, runtime) -> None:
         for p in self.parts():
             p.bind(tensors, runtime)
         for n in self._scale_names():
             self.scales[n] = take(tensors, n).contiguous()
+        for n in self.spec.unused:
+            if n in tensors:
+                take(tensors, n)
 
     def linears(self) -> list:
         return [lin for p in self.parts() for lin in p.linears()]

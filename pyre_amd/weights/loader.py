@@ -104,6 +104,8 @@ def check_against(specs: list[TensorSpec], index: dict, folder) -> None:
         if s.name not in index:
             if s.alias_of is not None and s.alias_of in index:
                 continue  # a tied tensor the file leaves out (pyre/loader.py:58-61)
+            if s.optional:
+                continue
             missing.append(s.name)
             continue
         if not s.fits(index[s.name][1]):

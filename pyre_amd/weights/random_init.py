@@ -35,7 +35,7 @@ def random_state(specs: list[TensorSpec], seed: int, std: float = 0.02, gain_std
     gen.manual_seed(seed)
     out: dict[str, torch.Tensor] = {}
     for s in specs:
-        if s.alias_of is not None:
+        if s.alias_of is not None or s.optional:
             continue
         shape = s.random_shape if s.random_shape is not None else s.shape
         if any(d is None for d in shape):

@@ -58,8 +58,10 @@ def test_manifest_names_shapes_and_caches():
     assert shapes["l0.mix.right.a1"] == (5, 48) and shapes["l0.mix.right.a2"] == (32, 5) and shapes["l0.mix.right.a2.b"] == (32,)
     assert shapes["l0.mix.right.norm"] == (24,) and shapes["l0.mlp.gate"] == (80, 48) and shapes["l0.mlp.down"] == (48, 80)
     assert shapes["l0.ls1"] == shapes["l0.ls2"] == shapes["l0.norm1b"] == shapes["l0.norm2b"] == (48,)
-    # the layer without a feed-forward has none of its tensors
-    assert "l1.norm1b" in shapes and not any(n.startswith(("l1.mlp", "l1.norm2", "l1.ls2")) for n in shapes)
+    # the layer without a feed-forward has none of its matrices; that half's norms and scale may be in a file, unread
+    optional = {s.name for s in model.tensor_specs() if s.optional}
+    assert "l1.norm1b" in shapes and not any(n.startswith("l1.mlp") for n in shapes)
+    assert optional == {"l1.norm2", "l1.norm2b", "l1.ls2"}
     assert "lm_head.weight" not in shapes
     kept = model.cache_specs()
     assert kept[0] == [PagedCacheSpec((PagedTensorSpec("k", (2, 24), 1), PagedTensorSpec("v", (2, 16), 1)), 20, 3),
@@ -107,3 +109,25 @@ def test_random_folder_loads_back(tmp_path):
     assert float(w["l0.mix.left.rel"].abs().max()) > 0.2   # the distance table is drawn wide enough to matter
     logits = P.forward(raw, w, [3, 1, 4, 1, 5])
     assert logits.shape == (5, 31) and bool(logits.isfinite().all())
+
+
+def test_norms_of_a_missing_feed_forward_may_be_in_the_file_or_not(tmp_path):
+    import torch
+    from safetensors.torch import load_file, save_file
+
+    from pyre_amd.weights import write_random_model
+    from pyre_amd.weights.loader import WeightsError, check_against, checkpoint_index
+
+    cfg = config_from_dict(M.SMALL)
+    write_random_model(tmp_path, cfg, seed=6)
+    specs = LayeredModel(get_architecture("Mafurax").build(cfg)).tensor_specs()
+    state = load_file(str(tmp_path / "model.safetensors"))
+    assert "l1.norm2" not in state
+    check_against(specs, checkpoint_index(tmp_path), tmp_path)
+    state.update({n: torch.ones(48, dtype=torch.bfloat16) for n in ("l1.norm2", "l1.norm2b", "l1.ls2")})
+    save_file(state, str(tmp_path / "model.safetensors"))
+    check_against(specs, checkpoint_index(tmp_path), tmp_path)
+    state["l1.mlp.gate"] = torch.ones(4, 48, dtype=torch.bfloat16)      # a matrix that no part names is still refused
+    save_file(state, str(tmp_path / "model.safetensors"))
+    with pytest.raises(WeightsError):
+        check_against(specs, checkpoint_index(tmp_path), tmp_path)
