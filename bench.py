@@ -221,9 +221,9 @@ def designs(args) -> dict:
                 "intermediate_size": sh["ff"], "vocab_size": sh["vocab"], "rope_theta": 1e6, "rms_norm_eps": 1e-6,
                 "tie_word_embeddings": True, "max_position_embeddings": 32768}
         left = {"heads": sh["heads"] // 2, "kv_heads": max(1, sh["kv_heads"] // 2), "dim": sh["head"], "vdim": sh["head"],
-                "scale": sh["head"] ** -0.5, "softcap": 30.0, "bias_max": 1024, "bias_rows": 32,
+                "scale": sh["head"] ** -0.5, "softcap": 50.0, "bias_max": 1024, "bias_rows": 32,
                 "mask": {"size": 1024, "keep_first": 4}}
-        right = {"heads": sh["heads"] // 2, "dim": sh["head"], "vdim": sh["head"], "tau": 16.0, "rank": 16}
+        right = {"heads": sh["heads"] // 2, "dim": sh["head"], "vdim": sh["head"], "tau": 8.0, "rank": 32}
         layer = {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0},
                  "mlp": {"kind": "dense", "ff": sh["ff"], "limit": 7.0}}
         mafurax = {"architecture": "Mafurax", "vocab": sh["vocab"], "width": sh["width"], "layers": [layer] * layers,

@@ -14,7 +14,7 @@ from pyre_amd.parts.base import (CappedAttentionSpec, PagedCacheSpec, PagedTenso
 from pyre_amd.parts.branch import BranchMixer
 
 #: rows of the distance table that the random-weights mode draws when a description leaves them to the file
-DEFAULT_BIAS_ROWS = 16
+DEFAULT_BIAS_ROWS = 32
 
 
 def distance_rows(rows: int, far: float) -> list[int]:

@@ -52,7 +52,7 @@ class ClippedGLU(FeedForward):
     def __init__(self, spec: ClippedGLUSpec):
         self.spec = spec
         self.gate_up = Linear(spec.hidden_size, 2 * spec.intermediate_size, "ffn.gate_up")
-        self.down = Linear(spec.intermediate_size, spec.hidden_size, "ffn.down")
+        self.down = Linear(spec.intermediate_size, spec.hidden_size, "glu.down")
 
     def tensor_specs(self) -> list[TensorSpec]:
         s, p = self.spec, self.spec.prefix

@@ -9,7 +9,7 @@ from pyre_amd.parts.base import GatedLinearAttentionSpec, StateCacheSpec, Tensor
 from pyre_amd.parts.branch import BranchMixer
 
 #: columns of the decay's low-rank product that the random-weights mode draws when a description leaves them to the file
-DEFAULT_RANK = 16
+DEFAULT_RANK = 8
 
 
 class GatedLinearAttention(BranchMixer):
