@@ -408,7 +408,34 @@ def test_greedy_generation_through_the_scheduler(graphs, folders):
         assert eng.graph_replays > 0
 
 
-@pytest.mark.parametrize("dtype,extra", [("float32", ("--page-size", "8", "--poison")), ("bfloat16", ())])
+def test_the_generate_program_as_a_process(folders, tmp_path):
+    """``bin/pyre_generate`` finds the design by the folder's config.json like any other: sampled tokens of a
+    process of its own against the plain implementation's greedy choice."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    folder, cfg, w = folders["wide"]
+    root = Path(__file__).resolve().parent.parent
+    out = tmp_path / "res.json"
+    proc = subprocess.run([sys.executable, str(root / "bin" / "pyre_generate"), "--model", str(folder), "--dtype", "float32",
+                           "--prompt-ids", "7,3,3,41,9,60,5", "--prompt-ids", "11", "--tokens", "12", "--num-blocks", "32",
+                           "--max-batch", "2", "--out", str(out)], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    res = json.loads(out.read_text())
+    assert res["dtype"] == "float32" and [len(g) for g in res["generated"]] == [12, 12]
+    for prompt, tokens in zip(res["prompts"], res["generated"]):
+        ids = list(prompt)
+        for k, tok in enumerate(tokens):
+            row = P.forward(cfg, w, ids)[-1]
+            twin = int(row.argmax())
+            if twin != tok:
+                margin = float((row[twin] - row[tok]) / row.abs().max())
+                assert margin < TOL["float32"], f"token {k} is {tok}, plainly {twin} (margin {margin:.2e})"
+            ids.append(tok)
+
+
+@pytest.mark.parametrize("dtype,extra", [("float32", ("--page-size", "8", "--poison")), ("bfloat16", ("--graphs",))])
 def test_trace_run_as_a_process(dtype, extra, folders, tmp_path):
     from test_trace_run_gpu import run_trace
 
