@@ -65,7 +65,7 @@ template <int CW, int XW, int RW, int EPI, int NL, int S>
 __global__ __launch_bounds__(64 * (XW * RW + NL)) void gemm_mid_kernel(const bf16* __restrict__ X, size_t ldx,
                                                                       const bf16* __restrict__ W, size_t ldw,
                                                                       void* __restrict__ out, int M, int N, int K,
-                                                                      int kper) {
+                                                                      int kper, GateShape act) {
   constexpr int BM = 32 * CW * XW, BW = BN * RW, ROWS = BW + BM, STAGE = ROWS * 128;
   constexpr int NWAVES = XW * RW + NL, LOADS = ROWS / 8;
   constexpr int PER = (LOADS + NWAVES - 1) / NWAVES;  // loads of 8 rows per wave and stage
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(64 * (XW * RW + NL)) void gemm_mid_kernel(const bf1
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float gate = acc[0][ct][4 * q + j], up = acc[1][ct][4 * q + j];
-          y[j] = gate / (1.f + __expf(-gate)) * up;
+          y[j] = gated_unit(gate, up, act);
         }
         bf16* dst = o + static_cast<size_t>(m) * inter + f;
         if (vec && f + 3 < inter) {
@@ -250,6 +250,7 @@ extern "C" int pyre_gemm_mid_supports(int M, int N, int K, long ldx, long ldw) {
 // out: float32 [ksplit][M][N].
 extern "C" int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long ldw, float* out, int M, int N,
                                   int K, int ksplit, int wide, hipStream_t stream) {
+  const GateShape act{};  // partial sums: no unit to finish
   if (int rc = check_mid("gemm_mid_bf16", X, W, M, N, K, ldx, ldw)) return rc;
   PYRE_REQUIRE(ksplit >= 1 && ksplit <= 64, "gemm_mid_bf16: ksplit=%d", ksplit);
   const int kper = ((K + ksplit - 1) / ksplit + BK - 1) / BK * BK;
@@ -266,35 +267,35 @@ extern "C" int pyre_gemm_mid_bf16(const void* X, long ldx, const void* W, long l
     const dim3 grid2((N + 2 * BN - 1) / (2 * BN), ksplit);
     if (M <= 32) {
       hipLaunchKernelGGL((gemm_mid_kernel<1, 1, 2, kPartials, 8, 6>), grid2, dim3(64 * 10), 0, stream, x,
-                         static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+                         static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper, act);
     } else if (M <= 64) {
       hipLaunchKernelGGL((gemm_mid_kernel<1, 2, 2, kPartials, 8, 5>), grid2, dim3(64 * 12), 0, stream, x,
-                         static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+                         static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper, act);
     } else if (M <= 128) {
       hipLaunchKernelGGL((gemm_mid_kernel<1, 4, 2, kPartials, 8, 4>), grid2, dim3(64 * 16), 0, stream, x,
-                         static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+                         static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper, act);
     } else if (M <= 192) {
       hipLaunchKernelGGL((gemm_mid_kernel<2, 3, 2, kPartials, 8, 3>), grid2, dim3(64 * 14), 0, stream, x,
-                         static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+                         static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper, act);
     } else {
       hipLaunchKernelGGL((gemm_mid_kernel<2, 4, 2, kPartials, 8, 3>), grid2, dim3(64 * 16), 0, stream, x,
-                         static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+                         static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper, act);
     }
   } else if (M > 192) {
     hipLaunchKernelGGL((gemm_mid_kernel<2, 4, 1, kPartials, 6, 3>), grid, dim3(64 * 10), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper, act);
   } else if (M > 128) {
     hipLaunchKernelGGL((gemm_mid_kernel<2, 3, 1, kPartials, 6, 4>), grid, dim3(64 * 9), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper, act);
   } else if (M <= 32) {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 1, 1, kPartials, 8, 6>), grid, dim3(64 * 9), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper, act);
   } else if (M <= 64) {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 2, 1, kPartials, 8, 5>), grid, dim3(64 * 10), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper, act);
   } else {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 4, 1, kPartials, 8, 4>), grid, dim3(64 * 12), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, N, K, kper, act);
   }
   return check_launch("gemm_mid_bf16");
 }
@@ -322,8 +323,8 @@ extern "C" int pyre_gemm_mid_silu_blocks(int M, int two_i) {
   return (two_i / 2 + f - 1) / f;
 }
 
-extern "C" int pyre_gemm_mid_silu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M,
-                                       int two_i, int K, hipStream_t stream) {
+static int mid_gated(const void* X, long ldx, const void* W, long ldw, void* out, int M, int two_i, int K, GateShape act,
+                     hipStream_t stream) {
   if (int rc = check_mid("gemm_mid_silu_bf16", X, W, M, two_i, K, ldx, ldw)) return rc;
   PYRE_REQUIRE(two_i % 2 == 0, "gemm_mid_silu_bf16: gate and up rows must be equally many");
   const int kper = (K + BK - 1) / BK * BK;
@@ -332,37 +333,48 @@ extern "C" int pyre_gemm_mid_silu_bf16(const void* X, long ldx, const void* W, l
   const bf16* w = static_cast<const bf16*>(W);
   if (M > 192) {
     hipLaunchKernelGGL((gemm_mid_kernel<2, 4, 2, kSiluMul, 8, 3>), grid, dim3(64 * 16), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper, act);
   } else if (M > 128) {
     hipLaunchKernelGGL((gemm_mid_kernel<2, 3, 2, kSiluMul, 8, 3>), grid, dim3(64 * 14), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper, act);
   } else if (M <= 32 && silu_features(M, two_i) == 128) {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 1, 4, kSiluMul, 8, 4>), grid, dim3(64 * 12), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper, act);
   } else if (M <= 64 && silu_features(M, two_i) == 128) {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 2, 4, kSiluMul, 8, 3>), grid, dim3(64 * 16), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper, act);
   } else if (M <= 32 && silu_features(M, two_i) == 96) {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 1, 3, kSiluMul, 8, 5>), grid, dim3(64 * 11), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper, act);
   } else if (M <= 32) {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 1, 2, kSiluMul, 8, 6>), grid, dim3(64 * 10), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper, act);
   } else if (M <= 64 && silu_features(M, two_i) == 96) {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 2, 3, kSiluMul, 8, 4>), grid, dim3(64 * 14), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper, act);
   } else if (M <= 64) {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 2, 2, kSiluMul, 8, 5>), grid, dim3(64 * 12), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper, act);
   } else if (M <= 96 && silu_features(M, two_i) == 96) {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 3, 3, kSiluMul, 6, 4>), grid, dim3(64 * 15), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper, act);
   } else if (silu_features(M, two_i) == 96) {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 4, 3, kSiluMul, 4, 3>), grid, dim3(64 * 16), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper, act);
   } else {
     hipLaunchKernelGGL((gemm_mid_kernel<1, 4, 2, kSiluMul, 8, 4>), grid, dim3(64 * 16), 0, stream, x,
-                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper);
+                       static_cast<size_t>(ldx), w, static_cast<size_t>(ldw), out, M, two_i, K, kper, act);
   }
   return check_launch("gemm_mid_silu_bf16");
+}
+
+extern "C" int pyre_gemm_mid_silu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M,
+                                       int two_i, int K, hipStream_t stream) {
+  return mid_gated(X, ldx, W, ldw, out, M, two_i, K, GateShape{}, stream);
+}
+
+// The same with another gated unit in the epilogue: g sigmoid(slope g) (u + shift), inputs clipped at `limit`.
+extern "C" int pyre_gemm_mid_glu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M, int two_i,
+                                      int K, float limit, float slope, float shift, hipStream_t stream) {
+  return mid_gated(X, ldx, W, ldw, out, M, two_i, K, GateShape{limit, slope, shift}, stream);
 }

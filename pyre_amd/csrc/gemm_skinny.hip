@@ -53,7 +53,8 @@ constexpr int kPad = 8;  // bf16 elements of padding per LDS row: rows land on d
 // What a wave does with its finished tiles. acc[t][mt]: lane (r, g) holds output rows
 // m = 16 mt + r, columns n0[t] + 4 g .. + 3.
 template <int RT, int MT, int EPI>
-__device__ inline void store_tiles(const f32x4 (&acc)[RT][MT], const int (&n0)[RT], void* out, int ks, int M, int N) {
+__device__ inline void store_tiles(const f32x4 (&acc)[RT][MT], const int (&n0)[RT], void* out, int ks, int M, int N,
+                                   GateShape act) {
   const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
   if (EPI == kPartials) {
     float* o = static_cast<float*>(out) + static_cast<size_t>(ks) * M * N;
@@ -86,7 +87,7 @@ __device__ inline void store_tiles(const f32x4 (&acc)[RT][MT], const int (&n0)[R
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float gate = acc[2 * p][mt][j], up = acc[2 * p + 1][mt][j];
-          y[j] = gate / (1.f + __expf(-gate)) * up;
+          y[j] = gated_unit(gate, up, act);
         }
         bf16* dst = o + static_cast<size_t>(m) * half + n;
         if (n + 3 < half && (half & 3) == 0) {
@@ -110,7 +111,7 @@ template <int RT, int MT, int EPI, int NWV>
 __global__ __launch_bounds__(64 * NWV) void gemm_skinny_kernel(const bf16* __restrict__ X, size_t ldx,
                                                               const bf16* __restrict__ W, size_t ldw,
                                                               void* __restrict__ out, int M, int N, int K,
-                                                              int kper) {
+                                                              int kper, GateShape act) {
   constexpr int NT = 64 * NWV;                    // threads
   constexpr int R = 16 * RT * NWV;                // rows of W per block
   constexpr int PR = kRun / 8;                    // 16-byte pieces of a row per run
@@ -201,7 +202,7 @@ __global__ __launch_bounds__(64 * NWV) void gemm_skinny_kernel(const bf16* __res
 #pragma unroll
   for (int t = 0; t < RT; ++t)
     n0[t] = EPI == kSiluMul ? blockIdx.x * (R / 2) + wave * 16 : blockIdx.x * R + (wave * RT + t) * 16;
-  store_tiles<RT, MT, EPI>(acc, n0, out, ks, M, N);
+  store_tiles<RT, MT, EPI>(acc, n0, out, ks, M, N, act);
 }
 
 // ---------------------------------------------------------------------------
@@ -216,7 +217,7 @@ template <int RT, int EPI>
 __global__ __launch_bounds__(64) void gemm_skinny_wave_kernel(const bf16* __restrict__ X, size_t ldx,
                                                               const bf16* __restrict__ W, size_t ldw,
                                                               void* __restrict__ out, int M, int N, int K,
-                                                              int kper) {
+                                                              int kper, GateShape act) {
   constexpr int U = kRun / 32;  // MFMA steps per run
   __shared__ __attribute__((aligned(16))) bf16 wl[RT][16][kRun + kPad];
   const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
@@ -279,15 +280,15 @@ __global__ __launch_bounds__(64) void gemm_skinny_wave_kernel(const bf16* __rest
       use(wb, xb);
     }
   }
-  store_tiles<RT, 1, EPI>(acc, n0, out, ks, M, N);
+  store_tiles<RT, 1, EPI>(acc, n0, out, ks, M, N, act);
 }
 
 template <int RT, int EPI, int NWV>
 int launch_skinny(int mt, dim3 grid, hipStream_t stream, const bf16* X, size_t ldx, const bf16* W, size_t ldw,
-                  void* out, int M, int N, int K, int kper) {
+                  void* out, int M, int N, int K, int kper, GateShape act = GateShape{}) {
 #define PYRE_LAUNCH_MT(MTV)                                                                                  \
   hipLaunchKernelGGL((gemm_skinny_kernel<RT, MTV, EPI, NWV>), grid, dim3(64 * NWV), 0, stream, X, ldx, W, ldw, \
-                     out, M, N, K, kper)
+                     out, M, N, K, kper, act)
   switch (mt) {
     case 1: PYRE_LAUNCH_MT(1); return 0;
     case 2: PYRE_LAUNCH_MT(2); return 0;
@@ -353,8 +354,19 @@ extern "C" int pyre_gemm_skinny_bf16(const void* X, long ldx, const void* W, lon
 }
 
 // W = [gate rows; up rows] (2I x K); out: bfloat16 [M][I] = silu(X gate^T) * (X up^T).
-extern "C" int pyre_gemm_skinny_silu_bf16(const void* X, long ldx, const void* W, long ldw, void* out,
-                                          int M, int two_i, int K, hipStream_t stream) {
+static int skinny_gated(const void* X, long ldx, const void* W, long ldw, void* out, int M, int two_i, int K, GateShape act,
+                        hipStream_t stream);
+extern "C" int pyre_gemm_skinny_silu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M, int two_i,
+                                          int K, hipStream_t stream) {
+  return skinny_gated(X, ldx, W, ldw, out, M, two_i, K, GateShape{}, stream);
+}
+// The same with another gated unit in the epilogue: g sigmoid(slope g) (u + shift), inputs clipped at `limit`.
+extern "C" int pyre_gemm_skinny_glu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M, int two_i,
+                                         int K, float limit, float slope, float shift, hipStream_t stream) {
+  return skinny_gated(X, ldx, W, ldw, out, M, two_i, K, GateShape{limit, slope, shift}, stream);
+}
+static int skinny_gated(const void* X, long ldx, const void* W, long ldw, void* out, int M, int two_i, int K, GateShape act,
+                        hipStream_t stream) {
   if (int rc = check_common("gemm_skinny_silu_bf16", M, two_i, K, ldx, ldw)) return rc;
   PYRE_REQUIRE(two_i % 2 == 0, "gemm_skinny_silu_bf16: gate and up rows must be equally many");
   const int mt = (M + 15) / 16;
@@ -364,13 +376,13 @@ extern "C" int pyre_gemm_skinny_silu_bf16(const void* X, long ldx, const void* W
   const bf16* w = static_cast<const bf16*>(W);
   if (mt == 1) {  // every wave on its own: measured 45 us against 50 on the 7B gate/up product (the other products gain nothing)
     hipLaunchKernelGGL((gemm_skinny_wave_kernel<2, kSiluMul>), dim3(tiles, 1), dim3(64), 0, stream, x, ldx, w, ldw,
-                       out, M, two_i, K, kper);
+                       out, M, two_i, K, kper, act);
     return check_launch("gemm_skinny_silu_bf16");
   }
   const dim3 grid((tiles + waves - 1) / waves, 1);
   int rc = 1;
   switch (waves) {
-#define PYRE_CASE(NWV) case NWV: rc = launch_skinny<2, kSiluMul, NWV>(mt, grid, stream, x, ldx, w, ldw, out, M, two_i, K, kper); break
+#define PYRE_CASE(NWV) case NWV: rc = launch_skinny<2, kSiluMul, NWV>(mt, grid, stream, x, ldx, w, ldw, out, M, two_i, K, kper, act); break
     PYRE_CASE(3); PYRE_CASE(4); PYRE_CASE(5); PYRE_CASE(6);
 #undef PYRE_CASE
   }

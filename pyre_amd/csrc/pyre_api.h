@@ -208,6 +208,13 @@ int pyre_feed_tokens(int* tokens, const int* src, const int* ids, int n, hipStre
 int pyre_sample(const float* logits, long row_stride, const float* temperature,
                 const float* uniform, int* out, int m, int vocab, hipStream_t stream);
 
+// The gate/up products with another gated unit in the epilogue: out = g sigmoid(slope g) (u + shift) with
+// g = min(X gate^T, limit), u = clamp(X up^T, -limit, limit) (limit <= 0: no clipping); shapes as the _silu_ forms.
+int pyre_gemm_skinny_glu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M, int two_i, int K,
+                              float limit, float slope, float shift, hipStream_t stream);
+int pyre_gemm_mid_glu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M, int two_i, int K,
+                           float limit, float slope, float shift, hipStream_t stream);
+
 // ---- layer norm around the residual stream, clipped gated activation, scaling (layernorm.hip) ----
 // resid += y, out = LN(resid) * gain, where y is the pending term (partial sums, bias) or, with
 // post_gain, LN(term; post_eps) * post_gain (* post_scale). rows: only these rows, resid untouched.

@@ -110,6 +110,20 @@ __device__ inline void store_from_float(void* p, int dt, size_t i, float v) {
   else static_cast<bf16*>(p)[i] = from_float<bf16>(v);
 }
 
+// The gated unit that a gate/up product may finish in its epilogue: g sigmoid(slope g) (u + shift) with
+// g = min(gate, limit), u = clamp(up, -limit, limit) (limit <= 0: no clipping). The defaults are the SiLU-gate;
+// the exponential is the hardware's (the result is rounded to bfloat16).
+struct GateShape {
+  float limit = 0.f, slope = 1.f, shift = 0.f;
+};
+__device__ inline float gated_unit(float gate, float up, GateShape a) {
+  if (a.limit > 0.f) {
+    gate = fminf(gate, a.limit);
+    up = fminf(fmaxf(up, -a.limit), a.limit);
+  }
+  return gate / (1.f + __expf(-a.slope * gate)) * (up + a.shift);
+}
+
 __device__ inline float wave_sum(float v) {
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);

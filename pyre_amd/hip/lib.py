@@ -11,7 +11,7 @@ from ctypes import c_float, c_int, c_long, c_void_p
 
 from pyre_amd.hip import build as _build
 
-ABI_VERSION = 24
+ABI_VERSION = 25
 
 
 class KernelError(RuntimeError):
@@ -53,6 +53,8 @@ _SIGNATURES = {
     "pyre_gemm_mid_silu_bf16": [P, L, P, L, P, I, I, I, P],
     "pyre_sample": [P, L, P, P, P, I, I, P],
     "pyre_feed_tokens": [P, P, P, I, P],
+    "pyre_gemm_skinny_glu_bf16": [P, L, P, L, P, I, I, I, F, F, F, P],
+    "pyre_gemm_mid_glu_bf16": [P, L, P, L, P, I, I, I, F, F, F, P],
     "pyre_add_layernorm": [P, P, I, I, L, P, I, P, I, P, I, F, P, I, P, I, P, I, I, F, P],
     "pyre_clipped_glu": [P, I, I, L, P, I, I, I, F, F, P],
     "pyre_scale": [P, L, F, P],

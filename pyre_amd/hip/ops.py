@@ -858,13 +858,20 @@ def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int
          w.shape[1], ksplit, _stream())
 
 
-def gemm_skinny_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, m: int) -> None:
-    """out[0:m] (bfloat16 [m, I]) = silu(x @ gate.T) * (x @ up.T) with w_gate_up = [gate; up]."""
+def gemm_skinny_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, m: int,
+                          unit: tuple[float, float, float] | None = None) -> None:
+    """out[0:m] (bfloat16 [m, I]) = silu(x @ gate.T) * (x @ up.T) with w_gate_up = [gate; up]. ``unit`` =
+    (limit, slope, shift): g * sigmoid(slope * g) * (u + shift) with g = min(gate, limit), u = clamp(up, -limit,
+    limit) instead (limit <= 0: no clipping)."""
     _skinny_common(x, w_gate_up, m)
     two_i = w_gate_up.shape[0]
     if (out.dtype != torch.bfloat16 or not out.is_contiguous() or not out.is_cuda or out.dim() != 2
             or out.shape[1] * 2 != two_i or out.shape[0] < m):
         raise KernelError("gemm_skinny_silu: out must be contiguous bfloat16 [>= m, I] on the GPU")
+    if unit is not None:
+        call("pyre_gemm_skinny_glu_bf16", x.data_ptr(), x.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
+             out.data_ptr(), m, two_i, w_gate_up.shape[1], *(float(v) for v in unit), _stream())
+        return
     call("pyre_gemm_skinny_silu_bf16", x.data_ptr(), x.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
          out.data_ptr(), m, two_i, w_gate_up.shape[1], _stream())
 
@@ -894,13 +901,19 @@ def gemm_mid_silu_blocks(m: int, two_i: int) -> int:
     return int(lib().pyre_gemm_mid_silu_blocks(m, two_i))
 
 
-def gemm_mid_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, m: int) -> None:
-    """out[0:m] (bfloat16 [m, I]) = silu(x @ gate.T) * (x @ up.T) with w_gate_up = [gate; up], 1 <= m <= 256."""
+def gemm_mid_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, m: int,
+                       unit: tuple[float, float, float] | None = None) -> None:
+    """out[0:m] (bfloat16 [m, I]) = silu(x @ gate.T) * (x @ up.T) with w_gate_up = [gate; up], 1 <= m <= 256;
+    ``unit`` as for :func:`gemm_skinny_silu_bf16`."""
     _skinny_common(x, w_gate_up, m)
     two_i = w_gate_up.shape[0]
     if (out.dtype != torch.bfloat16 or not out.is_contiguous() or not out.is_cuda or out.dim() != 2
             or out.shape[1] * 2 != two_i or out.shape[0] < m):
         raise KernelError("gemm_mid_silu: out must be contiguous bfloat16 [>= m, I] on the GPU")
+    if unit is not None:
+        call("pyre_gemm_mid_glu_bf16", x.data_ptr(), x.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
+             out.data_ptr(), m, two_i, w_gate_up.shape[1], *(float(v) for v in unit), _stream())
+        return
     call("pyre_gemm_mid_silu_bf16", x.data_ptr(), x.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
          out.data_ptr(), m, two_i, w_gate_up.shape[1], _stream())
 

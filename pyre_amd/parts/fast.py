@@ -187,8 +187,9 @@ def linear(lin, ctx, x, n, out):
     return Partials(buf.view(1, n, n_out), lin.bias)
 
 
-def gate_up_silu(lin, ctx, x, n, act) -> bool:
-    """silu(x gate^T) * (x up^T) in one kernel: the kernel that keeps all rows in a block for up to
+def gate_up_silu(lin, ctx, x, n, act, unit=None) -> bool:
+    """silu(x gate^T) * (x up^T) in one kernel (``unit`` = (limit, slope, shift): the gated unit
+    g sigmoid(slope g) (u + shift) with clipped inputs instead, in the same epilogues): the kernel that keeps all rows in a block for up to
     256 rows where one round of blocks holds the features, else the weight-streaming kernel for a
     decode step's few rows."""
     from pyre_amd.hip import ops
@@ -207,13 +208,13 @@ def gate_up_silu(lin, ctx, x, n, act) -> bool:
         mid = ctx.runtime.options.get("mid_gemm", True)
         fits = mid and ops.gemm_mid_supports(n, lin.out_features, lin.in_features, x.stride(0), lin.weight.stride(0))
         if fits and (ops.gemm_mid_silu_blocks(n, lin.out_features) <= ctx.runtime.compute_units or int(mid) == 2):
-            ops.gemm_mid_silu_bf16(x, lin.weight, act, n)
+            ops.gemm_mid_silu_bf16(x, lin.weight, act, n, unit)
             return True
     if n > FUSED_SILU_MAX_ROWS or not ctx.runtime.options.get("skinny_gemm", True):
         return False
     if not ops.gemm_skinny_supports(n, lin.out_features, lin.in_features, x.stride(0), lin.weight.stride(0)):
         return False
-    ops.gemm_skinny_silu_bf16(x, lin.weight, act, n)
+    ops.gemm_skinny_silu_bf16(x, lin.weight, act, n, unit)
     return True
 
 

@@ -74,6 +74,8 @@ class ClippedGLU(FeedForward):
     def forward(self, ctx, h):
         n = ctx.n_tokens
         act = ctx.workspace.get("ffn.act", (n, self.spec.intermediate_size), ctx.dtype)
-        gu = self.gate_up.forward(ctx, h, n)
-        ops.clipped_glu(gu, act, n, self.spec.limit, self.spec.slope)
+        # a step of few rows finishes the unit in the gate/up product's epilogue, as the SiLU-gate is finished
+        if not fast.gate_up_silu(self.gate_up, ctx, h, n, act, unit=(self.spec.limit, self.spec.slope, 1.0)):
+            gu = self.gate_up.forward(ctx, h, n)
+            ops.clipped_glu(gu, act, n, self.spec.limit, self.spec.slope)
         return self.down.forward(ctx, act, n)

@@ -381,6 +381,35 @@ def test_clipped_gated_unit():
     assert float((out.cpu().double() - P.clamped_glu(h, w, "f", {"limit": 0.7})).abs().max()) < 1e-5
 
 
+@pytest.mark.parametrize("rows", [1, 8, 40, 64, 100, 200])
+def test_clipped_gated_unit_in_the_gate_up_products_epilogue(rows):
+    """The decode step's gate/up product finishes the unit itself, as it finishes the SiLU-gate."""
+    from pyre_amd.hip import ops
+
+    g = torch.Generator().manual_seed(rows)
+    k, inter = 512, 384
+    x = (torch.randn(rows, k, generator=g) * 0.5).bfloat16()
+    w = (torch.randn(2 * inter, k, generator=g) * 0.08).bfloat16()
+    both = x.double() @ w.double().T
+    gate, up = both[:, :inter].clamp(max=0.9), both[:, inter:].clamp(-0.9, 0.9)
+    want = gate * torch.sigmoid(1.702 * gate) * (up + 1)
+    plain = both[:, :inter] * torch.sigmoid(both[:, :inter]) * both[:, inter:]
+    assert bool((both[:, :inter] > 0.9).any() and (both[:, inter:] < -0.9).any())
+    xd, wd = x.to("cuda:0"), w.to("cuda:0")
+    ran = 0
+    for name, supports, fn in (("skinny", ops.gemm_skinny_supports, ops.gemm_skinny_silu_bf16),
+                               ("mid", ops.gemm_mid_supports, ops.gemm_mid_silu_bf16)):
+        if rows > (64 if name == "skinny" else 256) or not supports(rows, 2 * inter, k, xd.stride(0), wd.stride(0)):
+            continue
+        out = torch.zeros(rows, inter, device="cuda:0", dtype=torch.bfloat16)
+        fn(xd, wd, out, rows, (0.9, 1.702, 1.0))
+        assert float((out.cpu().double() - want).abs().max()) < 1e-2 * float(want.abs().max()), name
+        fn(xd, wd, out, rows)                      # and the SiLU-gate is what it was
+        assert float((out.cpu().double() - plain).abs().max()) < 1e-2 * float(plain.abs().max()), name
+        ran += 1
+    assert ran
+
+
 # ----------------------------------------------------------------------------- the entry points
 
 
