@@ -7,6 +7,7 @@
 //
 //   s(i, j) = (q_i . k_j) * scale;   s <- cap * tanh(s / cap)  (cap > 0);   s <- s + bias[head][min(i - j, far)]
 //   i sees j  iff  j <= i and (window == 0 or i - j < window or j < keep_first)
+//                 and (chunk == 0 or i / chunk == j / chunk)      (chunks of positions counted from 0)
 //   out_i = gate_i * out_scale * sum_j softmax_j(s(i, .)) v_j
 //
 // `bias` is the table by distance that the host made of the model's buckets: [nq][far + 1] float32,
@@ -148,6 +149,13 @@ __device__ inline float tanh_by_exp(float x) {
   return copysignf((1.f - e) / (1.f + e), x);
 }
 
+// The first key that a query at `pos` sees, the kept first tokens aside.
+__device__ inline int first_seen(int pos, int window, int chunk) {
+  int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  if (chunk > 0) lo = max(lo, pos - pos % chunk);
+  return lo;
+}
+
 __device__ inline float shaped_score(float raw, float scale, float cap, const float* bias_row, int dist, int far) {
   float s = raw * scale;
   if (cap > 0.f) s = cap * tanh_by_exp(s / cap);
@@ -167,7 +175,7 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
     int out_ld, const float* __restrict__ gate, float out_scale, const int* __restrict__ tiles,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, int nq, int nkv, int dk, int dkp, int dv, int page_size, float scale, float cap,
-    const float* __restrict__ bias, int far, int window, int keep_first, int tab_lds, int bias_lds) {
+    const float* __restrict__ bias, int far, int window, int keep_first, int chunk, int tab_lds, int bias_lds) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // rows of keys and queries hold the even elements first, then the odd ones: a lane's operands of four
   // steps of the first product are then one 16-byte read
@@ -190,7 +198,7 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
 
   const bool live = active && c < ntok;
   const int hi = c < ntok ? pos0 + c : pos0;
-  const int lo = window > 0 ? max(0, hi - window + 1) : 0;
+  const int lo = first_seen(hi, window, chunk);
   const int keep = window > 0 ? keep_first : 0;
   const float* bias_row = bias ? bias + static_cast<size_t>(head) * (far + 1) : nullptr;
   for (int i = tid; i < tab_lds; i += kThreads) tab_s[i] = table[i];
@@ -224,7 +232,7 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
   float m = -INFINITY, l = 0.f;
 
   // the chunks that hold the kept first tokens which the window has passed, then the window's
-  const int lo_all = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int lo_all = first_seen(pos0, window, chunk);  // rises with the position: the tile's first token sees furthest back
   const int hi_all = pos0 + ntok - 1;
   const int kept_end = min(keep, lo_all);                        // keys 0 .. kept_end - 1 lie before every window
   const int n_first = kept_end > 0 ? (kept_end - 1) / kKeys + 1 : 0;
@@ -387,7 +395,7 @@ __global__ __launch_bounds__(kThreads) void attn_biased_single_kernel(
     int out_ld, const float* __restrict__ gate, float out_scale, const int* __restrict__ tokens,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale, float cap,
-    const float* __restrict__ bias, int far, int window, int keep_first, float* __restrict__ part) {
+    const float* __restrict__ bias, int far, int window, int keep_first, int chunk, float* __restrict__ part) {
   __shared__ __attribute__((aligned(16))) float qs[kMaxHead];
   __shared__ float sc[kSpan];
   __shared__ int row_s[kSpan];
@@ -397,7 +405,7 @@ __global__ __launch_bounds__(kThreads) void attn_biased_single_kernel(
   const int kvh = h / (nq / nkv);
   const int pos = positions[n];
   const int* table = block_table + static_cast<size_t>(seq_of_token[n]) * table_stride;
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = first_seen(pos, window, chunk);
   const int kept_end = window > 0 ? min(keep_first, lo) : 0;  // keys 0 .. kept_end - 1, then lo .. pos
   const float* bias_row = bias ? bias + static_cast<size_t>(h) * (far + 1) : nullptr;
   const int spans_first = (kept_end + kSpan - 1) / kSpan, spans_all = spans_first + (pos - lo) / kSpan + 1;
@@ -492,10 +500,10 @@ template <typename T>
 __global__ __launch_bounds__(kThreads) void attn_biased_join_kernel(
     const float* __restrict__ part, T* __restrict__ out, int out_ld, const float* __restrict__ gate, float out_scale,
     const int* __restrict__ tokens, const int* __restrict__ positions, int nq, int dv, int window, int keep_first,
-    int max_spans) {
+    int chunk, int max_spans) {
   const int n = tokens ? tokens[blockIdx.x] : blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int pos = positions[n];
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = first_seen(pos, window, chunk);
   const int kept_end = window > 0 ? min(keep_first, lo) : 0;
   const int spans = min(max_spans, (kept_end + kSpan - 1) / kSpan + (pos - lo) / kSpan + 1);
   const float* src = part + (static_cast<size_t>(blockIdx.x) * nq + h) * max_spans * (dv + 2);
@@ -555,10 +563,10 @@ extern "C" int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int d
                                      const float* gate, float out_scale, const int* tiles, int n_tiles,
                                      const int* positions, const int* seq_of_token, const int* block_table,
                                      int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale,
-                                     float cap, const float* bias, int far, int window, int keep_first,
+                                     float cap, const float* bias, int far, int window, int keep_first, int chunk,
                                      hipStream_t stream) {
   if (check_geometry("attn_biased_tile", nq, nkv, dk, dv, page_size)) return 1;
-  PYRE_REQUIRE(known_dtype(dt) && table_stride > 0 && window >= 0 && keep_first >= 0 && far >= 0, "attn_biased_tile: bad arguments");
+  PYRE_REQUIRE(known_dtype(dt) && table_stride > 0 && window >= 0 && keep_first >= 0 && far >= 0 && chunk >= 0, "attn_biased_tile: bad arguments");
   PYRE_REQUIRE(dk <= kTileMaxKeyHead, "attn_biased_tile: key heads of %d elements are more than %d", dk, kTileMaxKeyHead);
   if (n_tiles <= 0) return 0;
   const int hgroups = (nq / nkv + 3) / 4;
@@ -585,7 +593,7 @@ extern "C" int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int d
     hipLaunchKernelGGL((attn_biased_tile_kernel<T, NV, VEC>), grid, dim3(kThreads), lds, stream, static_cast<const T*>(q), \
                        static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), static_cast<T*>(out), out_ld, \
                        gate, out_scale, tiles, positions, seq_of_token, block_table, table_stride, nq, nkv, dk, dkp,  \
-                       dv, page_size, scale, cap, bias, far, window, keep_first, tab_lds, bias_lds);                 \
+                       dv, page_size, scale, cap, bias, far, window, keep_first, chunk, tab_lds, bias_lds);                 \
   } while (0)
 #define PYRE_TILE_NV(T, VEC)                \
   switch (nvp) {                            \
@@ -608,8 +616,9 @@ extern "C" int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int d
 
 // Spans of 128 keys that a token of such a launch can have: those of the kept first tokens and those
 // of the window (or of all `max_keys` keys that a block table holds).
-extern "C" int pyre_attn_biased_spans(int max_keys, int window, int keep_first) {
-  const int seen = window > 0 ? min(window, max_keys) : max_keys;
+extern "C" int pyre_attn_biased_spans(int max_keys, int window, int keep_first, int chunk) {
+  int seen = window > 0 ? min(window, max_keys) : max_keys;
+  if (chunk > 0) seen = min(seen, chunk);
   return (window > 0 ? (min(keep_first, max_keys) + kSpan - 1) / kSpan : 0) + (max(seen, 1) - 1) / kSpan + 1;
 }
 
@@ -617,10 +626,10 @@ extern "C" int pyre_attn_biased_single(const void* q, void* out, int out_ld, int
                                        const void* v_cache, const float* gate, float out_scale, const int* tokens,
                                        int n, const int* positions, const int* seq_of_token, const int* block_table,
                                        int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale,
-                                       float cap, const float* bias, int far, int window, int keep_first, float* part,
-                                       int max_spans, hipStream_t stream) {
+                                       float cap, const float* bias, int far, int window, int keep_first, int chunk,
+                                       float* part, int max_spans, hipStream_t stream) {
   if (check_geometry("attn_biased_single", nq, nkv, dk, dv, page_size)) return 1;
-  PYRE_REQUIRE(known_dtype(dt) && table_stride > 0 && window >= 0 && keep_first >= 0 && far >= 0, "attn_biased_single: bad arguments");
+  PYRE_REQUIRE(known_dtype(dt) && table_stride > 0 && window >= 0 && keep_first >= 0 && far >= 0 && chunk >= 0, "attn_biased_single: bad arguments");
   PYRE_REQUIRE(!part || (max_spans >= 1 && max_spans <= 65535), "attn_biased_single: %d spans are not a launch", max_spans);
   if (n <= 0) return 0;
   const dim3 grid(n, nq, part ? max_spans : 1);
@@ -629,7 +638,7 @@ extern "C" int pyre_attn_biased_single(const void* q, void* out, int out_ld, int
       hipLaunchKernelGGL((attn_biased_single_kernel<T, VEC>), grid, dim3(kThreads), 0, stream,                            \
                          static_cast<const T*>(q), static_cast<const T*>(k_cache), static_cast<const T*>(v_cache),        \
                          static_cast<T*>(out), out_ld, gate, out_scale, tokens, positions, seq_of_token, block_table,     \
-                         table_stride, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first, part))
+                         table_stride, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first, chunk, part))
   if (dk % 8 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0) {
     PYRE_SINGLE(true);
   } else {
@@ -639,6 +648,6 @@ extern "C" int pyre_attn_biased_single(const void* q, void* out, int out_ld, int
   if (part)
     PYRE_DISPATCH(dt, T,
         hipLaunchKernelGGL(attn_biased_join_kernel<T>, dim3(n, nq), dim3(kThreads), 0, stream, part, static_cast<T*>(out),
-                           out_ld, gate, out_scale, tokens, positions, nq, dv, window, keep_first, max_spans));
+                           out_ld, gate, out_scale, tokens, positions, nq, dv, window, keep_first, chunk, max_spans));
   return check_launch("attn_biased_single");
 }

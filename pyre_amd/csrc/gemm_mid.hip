@@ -373,8 +373,8 @@ extern "C" int pyre_gemm_mid_silu_bf16(const void* X, long ldx, const void* W, l
   return mid_gated(X, ldx, W, ldw, out, M, two_i, K, GateShape{}, stream);
 }
 
-// The same with another gated unit in the epilogue: g sigmoid(slope g) (u + shift), inputs clipped at `limit`.
+// The same with another gated unit in the epilogue: g sigmoid(slope (g + cubic g^3)) (u + shift), inputs clipped at `limit`.
 extern "C" int pyre_gemm_mid_glu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M, int two_i,
-                                      int K, float limit, float slope, float shift, hipStream_t stream) {
-  return mid_gated(X, ldx, W, ldw, out, M, two_i, K, GateShape{limit, slope, shift}, stream);
+                                      int K, float limit, float slope, float shift, float cubic, hipStream_t stream) {
+  return mid_gated(X, ldx, W, ldw, out, M, two_i, K, GateShape{limit, slope, shift, cubic}, stream);
 }

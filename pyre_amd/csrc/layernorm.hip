@@ -177,11 +177,11 @@ __global__ __launch_bounds__(THREADS) void add_layernorm_vec_kernel(
   }
 }
 
-// act[n, i] = g * sigmoid(slope * g) * (u + 1), g = min(gate[n, i], limit), u = clamp(up[n, i], -limit, limit);
+// act[n, i] = g * sigmoid(slope * (g + cubic g^3)) * (u + shift), g = min(gate[n, i], limit), u = clamp(up[n, i], -limit, limit);
 // gate = gu[:, :I], up = gu[:, I:], the partial sums added first. limit <= 0: no clipping.
 __global__ void clipped_glu_kernel(const void* __restrict__ gu, int gu_dt, int n_partials, size_t partial_stride,
                                    void* __restrict__ out, int out_dt, size_t total, int inter, float limit,
-                                   float slope) {
+                                   float slope, float shift, float cubic) {
   const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= total) return;
   const size_t n = i / inter, c = i % inter;
@@ -195,37 +195,38 @@ __global__ void clipped_glu_kernel(const void* __restrict__ gu, int gu_dt, int n
     g = fminf(g, limit);
     u = fminf(fmaxf(u, -limit), limit);
   }
-  store_from_float(out, out_dt, i, g / (1.f + expf(-slope * g)) * (u + 1.f));
+  store_from_float(out, out_dt, i, g / (1.f + expf(-slope * fmaf(cubic * g, g * g, g))) * (u + shift));
 }
 
-__device__ inline float clipped_unit(float g, float u, float limit, float slope) {
+__device__ inline float clipped_unit(float g, float u, float limit, float slope, float shift, float cubic) {
   if (limit > 0.f) {
     g = fminf(g, limit);
     u = fminf(fmaxf(u, -limit), limit);
   }
-  return g / (1.f + expf(-slope * g)) * (u + 1.f);
+  return g / (1.f + expf(-slope * fmaf(cubic * g, g * g, g))) * (u + shift);
 }
 
 // The same, four elements a thread (inter and the partial sums' stride are multiples of four).
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void clipped_glu_vec_kernel(const TI* __restrict__ gu, int n_partials, size_t partial_stride,
                                                               TO* __restrict__ out, size_t total4, int inter, float limit,
-                                                              float slope) {
+                                                              float slope, float shift, float cubic) {
   const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= total4) return;
   const int per_row = inter / 4;
   const size_t n = i / per_row, c = 4 * (i % per_row);
   const size_t gi = n * 2 * inter + c;
   const float4 g = sum_partials4(gu + gi, partial_stride, n_partials), u = sum_partials4(gu + gi + inter, partial_stride, n_partials);
-  Vec4<TO>::store(out + n * inter + c, float4{clipped_unit(g.x, u.x, limit, slope), clipped_unit(g.y, u.y, limit, slope),
-                                              clipped_unit(g.z, u.z, limit, slope), clipped_unit(g.w, u.w, limit, slope)});
+  Vec4<TO>::store(out + n * inter + c, float4{clipped_unit(g.x, u.x, limit, slope, shift, cubic), clipped_unit(g.y, u.y, limit, slope, shift, cubic),
+                                              clipped_unit(g.z, u.z, limit, slope, shift, cubic), clipped_unit(g.w, u.w, limit, slope, shift, cubic)});
 }
 
 // The same for many rows of bfloat16 in and out without partial sums to add: eight elements a thread,
 // loads that pass the caches (the rows are read once), the hardware's exponential and reciprocal (the
 // result is rounded to bfloat16 anyway).
 __global__ __launch_bounds__(256) void clipped_glu_stream_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out,
-                                                                 size_t total8, int inter, float limit, float slope) {
+                                                                 size_t total8, int inter, float limit, float slope,
+                                                                 float shift, float cubic) {
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
   const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= total8) return;
@@ -239,7 +240,7 @@ __global__ __launch_bounds__(256) void clipped_glu_stream_kernel(const bf16* __r
       gv = fminf(gv, limit);
       uv = fminf(fmaxf(uv, -limit), limit);
     }
-    return gv * __builtin_amdgcn_rcpf(1.f + __expf(-slope * gv)) * (uv + 1.f);
+    return gv * __builtin_amdgcn_rcpf(1.f + __expf(-slope * fmaf(cubic * gv, gv * gv, gv))) * (uv + shift);
   };
   u32x4 y;
 #pragma unroll
@@ -308,7 +309,8 @@ extern "C" int pyre_add_layernorm(float* resid, const void* delta, int delta_dt,
 }
 
 extern "C" int pyre_clipped_glu(const void* gu, int gu_dt, int n_partials, long partial_stride, void* out, int out_dt,
-                                int n, int inter, float limit, float slope, hipStream_t stream) {
+                                int n, int inter, float limit, float slope, float shift, float cubic,
+                                hipStream_t stream) {
   PYRE_REQUIRE(known_dtype(gu_dt) && known_dtype(out_dt), "clipped_glu: unknown dtype");
   PYRE_REQUIRE(n_partials >= 1 && inter > 0, "clipped_glu: bad sizes");
   if (n <= 0) return 0;
@@ -316,7 +318,7 @@ extern "C" int pyre_clipped_glu(const void* gu, int gu_dt, int n_partials, long 
       reinterpret_cast<uintptr_t>(gu) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
     const size_t total8 = static_cast<size_t>(n) * (inter / 8);
     hipLaunchKernelGGL(clipped_glu_stream_kernel, dim3((total8 + 255) / 256), dim3(256), 0, stream,
-                       static_cast<const bf16*>(gu), static_cast<bf16*>(out), total8, inter, limit, slope);
+                       static_cast<const bf16*>(gu), static_cast<bf16*>(out), total8, inter, limit, slope, shift, cubic);
     return check_launch("clipped_glu");
   }
   if (inter % 4 == 0 && partial_stride % 4 == 0 && reinterpret_cast<uintptr_t>(gu) % 16 == 0 &&
@@ -325,12 +327,12 @@ extern "C" int pyre_clipped_glu(const void* gu, int gu_dt, int n_partials, long 
     PYRE_DISPATCH(gu_dt, TI, PYRE_DISPATCH(out_dt, TO,
         hipLaunchKernelGGL((clipped_glu_vec_kernel<TI, TO>), dim3((total4 + 255) / 256), dim3(256), 0, stream,
                            static_cast<const TI*>(gu), n_partials, static_cast<size_t>(partial_stride),
-                           static_cast<TO*>(out), total4, inter, limit, slope)));
+                           static_cast<TO*>(out), total4, inter, limit, slope, shift, cubic)));
     return check_launch("clipped_glu");
   }
   const size_t total = static_cast<size_t>(n) * inter;
   hipLaunchKernelGGL(clipped_glu_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, gu, gu_dt, n_partials,
-                     static_cast<size_t>(partial_stride), out, out_dt, total, inter, limit, slope);
+                     static_cast<size_t>(partial_stride), out, out_dt, total, inter, limit, slope, shift, cubic);
   return check_launch("clipped_glu");
 }
 

@@ -208,12 +208,12 @@ int pyre_feed_tokens(int* tokens, const int* src, const int* ids, int n, hipStre
 int pyre_sample(const float* logits, long row_stride, const float* temperature,
                 const float* uniform, int* out, int m, int vocab, hipStream_t stream);
 
-// The gate/up products with another gated unit in the epilogue: out = g sigmoid(slope g) (u + shift) with
+// The gate/up products with another gated unit in the epilogue: out = g sigmoid(slope (g + cubic g^3)) (u + shift) with
 // g = min(X gate^T, limit), u = clamp(X up^T, -limit, limit) (limit <= 0: no clipping); shapes as the _silu_ forms.
 int pyre_gemm_skinny_glu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M, int two_i, int K,
-                              float limit, float slope, float shift, hipStream_t stream);
+                              float limit, float slope, float shift, float cubic, hipStream_t stream);
 int pyre_gemm_mid_glu_bf16(const void* X, long ldx, const void* W, long ldw, void* out, int M, int two_i, int K,
-                           float limit, float slope, float shift, hipStream_t stream);
+                           float limit, float slope, float shift, float cubic, hipStream_t stream);
 
 // ---- layer norm around the residual stream, clipped gated activation, scaling (layernorm.hip) ----
 // resid += y, out = LN(resid) * gain, where y is the pending term (partial sums, bias) or, with
@@ -223,9 +223,9 @@ int pyre_add_layernorm(float* resid, const void* delta, int delta_dt, int n_part
                        const void* post_scale, int post_scale_dt, float post_eps, const void* gain,
                        int gain_dt, void* out, int out_dt, const int* rows, int n, int hidden, float eps,
                        hipStream_t stream);
-// out[n, i] = g sigmoid(slope g) (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit); gu = [gate | up].
+// out[n, i] = g sigmoid(slope (g + cubic g^3)) (u + shift), g = min(gate, limit), u = clamp(up, -limit, limit); gu = [gate | up].
 int pyre_clipped_glu(const void* gu, int gu_dt, int n_partials, long partial_stride, void* out, int out_dt,
-                     int n, int inter, float limit, float slope, hipStream_t stream);
+                     int n, int inter, float limit, float slope, float shift, float cubic, hipStream_t stream);
 int pyre_scale(float* x, long total, float s, hipStream_t stream);
 
 // ---- attention with capped scores, a bias by distance and kept first tokens (attention_biased.hip) ----
@@ -235,25 +235,26 @@ int pyre_unit_qkv_write(const void* proj, int proj_dt, int n_partials, long part
                         void* q_out, int q_dt, void* k_cache, void* v_cache, int cache_dt, float* gate_out,
                         const int* slots, int n, int nq, int nkv, int dk, int dv, int page_size,
                         int unit_norm, float eps, int write_kv, hipStream_t stream);
+// chunk > 0: a query sees only the keys of its own run of `chunk` positions (runs counted from position 0).
 // tiles: [n_tiles][2] = (first token, count <= 32). bias: float32 [nq][far + 1] by distance, or null.
 // gate: float32 [tokens][nq] or null. out rows are out_ld elements apart; head h writes columns h dv ...
 int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int dt, const void* k_cache, const void* v_cache,
                           const float* gate, float out_scale, const int* tiles, int n_tiles,
                           const int* positions, const int* seq_of_token, const int* block_table,
                           int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale,
-                          float cap, const float* bias, int far, int window, int keep_first,
+                          float cap, const float* bias, int far, int window, int keep_first, int chunk,
                           hipStream_t stream);
 // tokens: the n tokens of the flat batch to attend for (null: 0..n-1), a block per token and head.
 int pyre_attn_biased_single(const void* q, void* out, int out_ld, int dt, const void* k_cache,
                             const void* v_cache, const float* gate, float out_scale, const int* tokens,
                             int n, const int* positions, const int* seq_of_token, const int* block_table,
                             int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale,
-                            float cap, const float* bias, int far, int window, int keep_first, float* part,
-                            int max_spans, hipStream_t stream);
+                            float cap, const float* bias, int far, int window, int keep_first, int chunk,
+                            float* part, int max_spans, hipStream_t stream);
 // part: scratch of n * nq * max_spans * (dv + 2) floats, max_spans = pyre_attn_biased_spans(the most keys a
 // block table holds, window, keep_first): a block then takes one span of 128 keys and a second kernel joins
 // them in their order; null: a block takes all spans of its token and head in turn.
-int pyre_attn_biased_spans(int max_keys, int window, int keep_first);
+int pyre_attn_biased_spans(int max_keys, int window, int keep_first, int chunk);
 
 // ---- gated linear attention (linear_attention.hip) ----
 // proj columns from col0 on: q, k (heads dk each), v, g (heads dv each), the low-rank input (rank).
@@ -272,5 +273,44 @@ int pyre_gla_chunks(const float* x, float* scratch, float* state, float* o, cons
                     int n_tokens, int n_seqs, int max_tokens, int heads, int dk, int dv, float qscale, hipStream_t stream);
 int pyre_gla_finish(const float* o, const float* x, const void* gain, int gain_dt, float eps, float out_scale,
                     void* out, int out_dt, int out_ld, int n, int heads, int dk, int dv, hipStream_t stream);
+
+// ---- a norm without statistics and the squashing of logits (tanh_norm.hip) ----
+// resid += a_scale (sum of a's partial sums + a_bias) + b_scale (the same of b); out = tanh(alpha resid) gain + shift.
+// a, b: pending terms or null (b only with a); alpha: one element; shift may be null; alpha, gain and shift share
+// param_dt. rows: only these rows, into a dense output, resid untouched.
+int pyre_add_tanhnorm(float* resid, const void* a, int a_dt, int a_count, long a_stride, const void* a_bias,
+                      int a_bias_dt, float a_scale, const void* b, int b_dt, int b_count, long b_stride,
+                      const void* b_bias, int b_bias_dt, float b_scale, const void* alpha, const void* gain,
+                      const void* shift, int param_dt, void* out, int out_dt, const int* rows, int n, int hidden,
+                      hipStream_t stream);
+// x <- cap tanh(x / cap), float32 in place.
+int pyre_softcap(float* x, long total, float cap, hipStream_t stream);
+
+// ---- between the input product and the attention kernels (latent.hip) ----
+// proj columns from col0 on: nq query heads and nkv key heads of d; bias over these columns or null. The first rot
+// elements of every head are turned by position (cos_t, sin_t: float32 [positions][rot / 2]); queries to
+// q_out [n, nq d], turned keys to k_cache and the keys as they were to v_cache (both [pages, nkv, page, d]).
+int pyre_rope_tied_write(const void* proj, int proj_dt, int n_partials, long partial_stride, int ld, int col0,
+                         const void* bias, int bias_dt, void* q_out, int q_dt, void* k_cache, void* v_cache,
+                         int cache_dt, const float* cos_t, const float* sin_t, int rot, const int* positions,
+                         const int* slots, int n, int nq, int nkv, int d, int page_size, int write_kv,
+                         hipStream_t stream);
+// proj columns from col0 on: q_width of queries, then (write) rank of the compressed row, which is stored divided
+// by its root mean square and times gain in c_cache [pages, 1, page, rank].
+int pyre_latent_write(const void* proj, int proj_dt, int n_partials, long partial_stride, int ld, int col0,
+                      void* q_out, int q_dt, void* c_cache, int cache_dt, const void* gain, int gain_dt, float eps,
+                      const int* slots, int n, int q_width, int rank, int page_size, int write, hipStream_t stream);
+// out[n, h, :] = x[n, h, :] w[h], w [heads, din, dout]; rows of x and out are x_ld and out_ld elements apart; one
+// element type for all three.
+int pyre_head_matmul(const void* x, int x_ld, const void* w, void* out, int out_ld, int dt, int n, int heads, int din,
+                     int dout, hipStream_t stream);
+
+// ---- a mixture of experts with a sigmoid router (moe.hip) ----
+// gates[n, experts] float32: s / (sum of the chosen s + 1e-20) for the `top` experts of largest s = sigmoid(z), else 0.
+int pyre_route_topk(const void* z, int z_dt, int n_partials, long partial_stride, const void* bias, int bias_dt,
+                    float* gates, int n, int experts, int top, hipStream_t stream);
+// out[n, e ff + j] = gates[n, e] max(up, 0)^2 for e < experts, max(up, 0)^2 for the shared_ff columns behind them.
+int pyre_expert_act(const void* up, int up_dt, int n_partials, long partial_stride, const float* gates, void* out,
+                    int out_dt, int n, int experts, int ff, int shared_ff, hipStream_t stream);
 
 }  // extern "C"

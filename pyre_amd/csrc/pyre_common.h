@@ -110,18 +110,19 @@ __device__ inline void store_from_float(void* p, int dt, size_t i, float v) {
   else static_cast<bf16*>(p)[i] = from_float<bf16>(v);
 }
 
-// The gated unit that a gate/up product may finish in its epilogue: g sigmoid(slope g) (u + shift) with
+// The gated unit that a gate/up product may finish in its epilogue: g sigmoid(slope (g + cubic g^3)) (u + shift) with
 // g = min(gate, limit), u = clamp(up, -limit, limit) (limit <= 0: no clipping). The defaults are the SiLU-gate;
+// slope 2 sqrt(2 / pi) with cubic 0.044715 is the tanh form of GELU, since (1 + tanh z) / 2 = sigmoid(2 z);
 // the exponential is the hardware's (the result is rounded to bfloat16).
 struct GateShape {
-  float limit = 0.f, slope = 1.f, shift = 0.f;
+  float limit = 0.f, slope = 1.f, shift = 0.f, cubic = 0.f;
 };
 __device__ inline float gated_unit(float gate, float up, GateShape a) {
   if (a.limit > 0.f) {
     gate = fminf(gate, a.limit);
     up = fminf(fmaxf(up, -a.limit), a.limit);
   }
-  return gate / (1.f + __expf(-a.slope * gate)) * (up + a.shift);
+  return gate / (1.f + __expf(-a.slope * fmaf(a.cubic * gate, gate * gate, gate))) * (up + a.shift);
 }
 
 __device__ inline float wave_sum(float v) {

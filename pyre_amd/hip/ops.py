@@ -83,6 +83,10 @@ class Partials:
     #: a norm (and layer scale) that the term goes through before it is added: only a norm
     #: that says so takes such a term (:func:`add_layernorm`)
     post: "PostNorm | None" = None
+    #: a factor on the whole term (sums and bias), and another term to be added with it (a layer whose
+    #: mixer and feed-forward read the same rows hands on both): only a norm that says so takes them
+    scale: float = 1.0
+    more: "Partials | None" = None
 
     def __post_init__(self) -> None:
         if self.data.dim() != 3 or not self.data.is_contiguous():
@@ -144,8 +148,8 @@ def add_rmsnorm(resid: torch.Tensor, delta: Partials | None, gain: torch.Tensor,
     if delta is not None:
         if delta.rows < resid.shape[0]:
             raise KernelError("add_rmsnorm: delta has fewer rows than the residual")
-        if delta.post is not None:
-            raise KernelError("add_rmsnorm: a term that is to be normed before it is added is not taken")
+        if delta.post is not None or delta.scale != 1.0 or delta.more is not None:
+            raise KernelError("add_rmsnorm: a term that is normed or scaled before it is added, or comes with another, is not taken")
         d = delta._args(hidden)
     else:
         d = (None, 0, 0, 0, None, 0)
@@ -175,6 +179,8 @@ def add_layernorm(resid: torch.Tensor, delta: Partials | None, gain: torch.Tenso
     if delta is not None:
         if delta.rows < resid.shape[0]:
             raise KernelError("add_layernorm: delta has fewer rows than the residual")
+        if delta.scale != 1.0 or delta.more is not None:
+            raise KernelError("add_layernorm: a term that is scaled before it is added, or comes with another, is not taken")
         d = delta._args(hidden)
         if delta.post is not None:
             pn = delta.post
@@ -192,9 +198,14 @@ def add_layernorm(resid: torch.Tensor, delta: Partials | None, gain: torch.Tenso
          dtype_code(out), _ptr(rows), n, hidden, float(eps), _stream())
 
 
-def clipped_glu(gu: Partials, out: torch.Tensor, n: int, limit: float, slope: float) -> None:
-    """out[n, i] = g * sigmoid(slope * g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit),
-    gate = gu[:, :I], up = gu[:, I:] (``limit`` <= 0: no clipping)."""
+#: slope and cubic term that make g sigmoid(slope (g + cubic g^3)) the tanh form of GELU: (1 + tanh z) / 2 = sigmoid(2 z)
+GELU_TANH_SLOPE, GELU_TANH_CUBIC = 2.0 * (2.0 / 3.141592653589793) ** 0.5, 0.044715
+
+
+def clipped_glu(gu: Partials, out: torch.Tensor, n: int, limit: float, slope: float, shift: float = 1.0,
+                cubic: float = 0.0) -> None:
+    """out[n, i] = g * sigmoid(slope * (g + cubic g^3)) * (u + shift) with g = min(gate, limit),
+    u = clamp(up, -limit, limit), gate = gu[:, :I], up = gu[:, I:] (``limit`` <= 0: no clipping)."""
     _dev(gu.data, out)
     inter = out.shape[-1]
     if gu.width != 2 * inter or gu.rows < n or out.shape[0] < n:
@@ -203,7 +214,7 @@ def clipped_glu(gu: Partials, out: torch.Tensor, n: int, limit: float, slope: fl
         raise KernelError("clipped_glu: a pending bias is not supported")
     _contig("out", out)
     call("pyre_clipped_glu", gu.data.data_ptr(), dtype_code(gu.data), gu.count, gu.stride, out.data_ptr(),
-         dtype_code(out), n, inter, float(limit), float(slope), _stream())
+         dtype_code(out), n, inter, float(limit), float(slope), float(shift), float(cubic), _stream())
 
 
 def scale_(x: torch.Tensor, s: float) -> None:
@@ -277,7 +288,7 @@ def _attn_biased_common(q, out, k_cache, v_cache, gate, positions, seq_of_token,
 
 
 def attn_biased_tile(q, out, k_cache, v_cache, gate, out_scale, tiles, n_tiles, positions, seq_of_token,
-                     block_table, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first) -> None:
+                     block_table, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first, chunk: int = 0) -> None:
     """Prompt portions of the capped, biased attention; ``tiles`` is int32 [n_tiles, 2] = (first token, count <= 32)."""
     _attn_biased_common(q, out, k_cache, v_cache, gate, positions, seq_of_token, block_table, bias, far,
                         nq, nkv, dk, dv, page_size)
@@ -285,19 +296,19 @@ def attn_biased_tile(q, out, k_cache, v_cache, gate, out_scale, tiles, n_tiles, 
     call("pyre_attn_biased_tile", q.data_ptr(), out.data_ptr(), out.stride(0), dtype_code(q), k_cache.data_ptr(),
          v_cache.data_ptr(), _ptr(gate), float(out_scale), tiles.data_ptr(), n_tiles, positions.data_ptr(),
          seq_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0), nq, nkv, dk, dv, page_size,
-         float(scale), float(cap), _ptr(bias), int(far), int(window), int(keep_first), _stream())
+         float(scale), float(cap), _ptr(bias), int(far), int(window), int(keep_first), int(chunk), _stream())
 
 
-def attn_biased_spans(table_width: int, page_size: int, window: int, keep_first: int) -> int:
+def attn_biased_spans(table_width: int, page_size: int, window: int, keep_first: int, chunk: int = 0) -> int:
     """Spans of 128 keys that a token can have when its block table is ``table_width`` pages wide."""
     from pyre_amd.hip.lib import lib
 
-    return int(lib().pyre_attn_biased_spans(max(1, table_width * page_size), int(window), int(keep_first)))
+    return int(lib().pyre_attn_biased_spans(max(1, table_width * page_size), int(window), int(keep_first), int(chunk)))
 
 
 def attn_biased_single(q, out, k_cache, v_cache, gate, out_scale, tokens, n, positions, seq_of_token,
                        block_table, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first,
-                       scratch: torch.Tensor | None = None) -> None:
+                       scratch: torch.Tensor | None = None, chunk: int = 0) -> None:
     """The same for ``n`` tokens one by one (``tokens``: which of the flat batch, None: the first n). ``scratch``
     (float32, ``n * nq * attn_biased_spans(...) * (dv + 2)`` elements): a block per span of 128 keys and a second
     kernel that joins them, instead of a block per token and head that takes its spans in turn."""
@@ -308,13 +319,13 @@ def attn_biased_single(q, out, k_cache, v_cache, gate, out_scale, tokens, n, pos
     spans = 0
     if scratch is not None:
         _dev(scratch)
-        spans = attn_biased_spans(block_table.shape[1], page_size, window, keep_first)
+        spans = attn_biased_spans(block_table.shape[1], page_size, window, keep_first, chunk)
         if scratch.dtype != torch.float32 or not scratch.is_contiguous() or scratch.numel() < n * nq * spans * (dv + 2):
             raise KernelError(f"attn_biased_single: scratch of {n * nq * spans * (dv + 2)} float32 elements needed")
     call("pyre_attn_biased_single", q.data_ptr(), out.data_ptr(), out.stride(0), dtype_code(q), k_cache.data_ptr(),
          v_cache.data_ptr(), _ptr(gate), float(out_scale), _ptr(tokens), n, positions.data_ptr(),
          seq_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0), nq, nkv, dk, dv, page_size,
-         float(scale), float(cap), _ptr(bias), int(far), int(window), int(keep_first), _ptr(scratch), spans, _stream())
+         float(scale), float(cap), _ptr(bias), int(far), int(window), int(keep_first), int(chunk), _ptr(scratch), spans, _stream())
 
 
 GLA_MAX_RANK = 512     #: the widest low-rank input of the decay (linear_attention.hip)
@@ -858,11 +869,22 @@ def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int
          w.shape[1], ksplit, _stream())
 
 
+def _gate_shape(unit) -> tuple[float, float, float, float]:
+    """(limit, slope, shift, cubic) of the gated unit g sigmoid(slope (g + cubic g^3)) (u + shift); a unit given
+    with three numbers has no cubic term."""
+    vals = [float(v) for v in unit]
+    if len(vals) == 3:
+        vals.append(0.0)
+    if len(vals) != 4:
+        raise KernelError("a gated unit is (limit, slope, shift[, cubic])")
+    return tuple(vals)
+
+
 def gemm_skinny_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, m: int,
                           unit: tuple[float, float, float] | None = None) -> None:
     """out[0:m] (bfloat16 [m, I]) = silu(x @ gate.T) * (x @ up.T) with w_gate_up = [gate; up]. ``unit`` =
-    (limit, slope, shift): g * sigmoid(slope * g) * (u + shift) with g = min(gate, limit), u = clamp(up, -limit,
-    limit) instead (limit <= 0: no clipping)."""
+    (limit, slope, shift[, cubic]): g * sigmoid(slope * (g + cubic g^3)) * (u + shift) with g = min(gate, limit),
+    u = clamp(up, -limit, limit) instead (limit <= 0: no clipping)."""
     _skinny_common(x, w_gate_up, m)
     two_i = w_gate_up.shape[0]
     if (out.dtype != torch.bfloat16 or not out.is_contiguous() or not out.is_cuda or out.dim() != 2
@@ -870,7 +892,7 @@ def gemm_skinny_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.T
         raise KernelError("gemm_skinny_silu: out must be contiguous bfloat16 [>= m, I] on the GPU")
     if unit is not None:
         call("pyre_gemm_skinny_glu_bf16", x.data_ptr(), x.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
-             out.data_ptr(), m, two_i, w_gate_up.shape[1], *(float(v) for v in unit), _stream())
+             out.data_ptr(), m, two_i, w_gate_up.shape[1], *_gate_shape(unit), _stream())
         return
     call("pyre_gemm_skinny_silu_bf16", x.data_ptr(), x.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
          out.data_ptr(), m, two_i, w_gate_up.shape[1], _stream())
@@ -912,7 +934,7 @@ def gemm_mid_silu_bf16(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tens
         raise KernelError("gemm_mid_silu: out must be contiguous bfloat16 [>= m, I] on the GPU")
     if unit is not None:
         call("pyre_gemm_mid_glu_bf16", x.data_ptr(), x.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
-             out.data_ptr(), m, two_i, w_gate_up.shape[1], *(float(v) for v in unit), _stream())
+             out.data_ptr(), m, two_i, w_gate_up.shape[1], *_gate_shape(unit), _stream())
         return
     call("pyre_gemm_mid_silu_bf16", x.data_ptr(), x.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
          out.data_ptr(), m, two_i, w_gate_up.shape[1], _stream())
@@ -935,3 +957,167 @@ def read_bandwidth(device: str = "cuda:0", gib: float = 2.0, blocks: int = 4096,
             call("pyre_read_probe", buf.data_ptr(), n, blocks, sink.data_ptr(), _stream())
         torch.cuda.synchronize()
     return n * repeats / (time.perf_counter() - t) / 1e9
+
+
+def add_tanhnorm(resid: torch.Tensor, delta: Partials | None, alpha: torch.Tensor, gain: torch.Tensor,
+                 shift: torch.Tensor | None, out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
+    """resid += delta (its partial sums and bias, times its ``scale``; the same for ``delta.more``, if any);
+    out = tanh(alpha * resid) * gain + shift: a norm that takes no statistic of the row. ``alpha`` holds one
+    number and shares its element type with ``gain`` and ``shift``.
+
+    With ``rows`` only those rows are normed, into ``out[0:len(rows)]``, and ``resid`` is left as it was."""
+    _dev(resid, alpha, gain, shift, out, rows)
+    hidden = resid.shape[-1]
+    if resid.dtype != torch.float32 or resid.dim() != 2:
+        raise KernelError("add_tanhnorm: the residual stream is float32 [N, H]")
+    n = resid.shape[0] if rows is None else rows.numel()
+    if out.shape[-1] != hidden or out.shape[0] < n or gain.numel() != hidden or alpha.numel() != 1 or \
+            (shift is not None and shift.numel() != hidden):
+        raise KernelError("add_tanhnorm: shapes of out / alpha / gain / shift do not fit the residual")
+    if alpha.dtype != gain.dtype or (shift is not None and shift.dtype != gain.dtype):
+        raise KernelError("add_tanhnorm: alpha, gain and shift share one element type")
+    _contig("resid", resid), _contig("out", out), _contig("gain", gain)
+    if shift is not None:
+        _contig("shift", shift)
+    if rows is not None:
+        _i32("rows", rows)
+    terms = []
+    t = delta
+    while t is not None:
+        if t.rows < resid.shape[0]:
+            raise KernelError("add_tanhnorm: a pending term has fewer rows than the residual")
+        if t.post is not None:
+            raise KernelError("add_tanhnorm: a term that is to be normed before it is added is not taken")
+        terms.append((*t._args(hidden), float(t.scale)))
+        t = t.more
+    if len(terms) > 2:
+        raise KernelError("add_tanhnorm: at most two pending terms")
+    while len(terms) < 2:
+        terms.append((None, 0, 0, 0, None, 0, 1.0))
+    call("pyre_add_tanhnorm", resid.data_ptr(), *terms[0], *terms[1], alpha.data_ptr(), gain.data_ptr(), _ptr(shift),
+         dtype_code(gain), out.data_ptr(), dtype_code(out), _ptr(rows), n, hidden, _stream())
+
+
+def softcap_(x: torch.Tensor, cap: float) -> None:
+    """x <- cap * tanh(x / cap) in place (contiguous float32)."""
+    _dev(x)
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelError("softcap_: contiguous float32 expected")
+    call("pyre_softcap", x.data_ptr(), x.numel(), float(cap), _stream())
+
+
+def rope_tied_write(proj: Partials, col0: int, q_out: torch.Tensor, k_cache: torch.Tensor | None,
+                    v_cache: torch.Tensor | None, cos: torch.Tensor | None, sin: torch.Tensor | None, rot: int,
+                    positions: torch.Tensor, slots: torch.Tensor | None, n: int, nq: int, nkv: int, d: int,
+                    page_size: int) -> None:
+    """Finish a step's input product from column ``col0`` on (``nq`` query heads, then ``nkv`` key heads, of ``d``;
+    ``proj.bias`` over these columns): the first ``rot`` elements of every head turned by position (element e with
+    e + rot/2, ``cos`` / ``sin`` float32 [positions, rot/2]), queries to ``q_out [N, nq*d]``, the turned keys to
+    ``k_cache`` and the keys as projected to ``v_cache`` (both ``[pages, nkv, page, d]``) at ``slots``."""
+    _dev(proj.data, proj.bias, q_out, k_cache, v_cache, cos, sin, positions, slots)
+    width = (nq + nkv) * d
+    if col0 < 0 or col0 + width > proj.width:
+        raise KernelError(f"columns {col0}..{col0 + width} lie outside the product's {proj.width}")
+    if proj.bias is not None and proj.bias.numel() != width:
+        raise KernelError(f"rope_tied_write: the bias has {proj.bias.numel()} entries, {width} expected")
+    if proj.rows < n or q_out.numel() < n * nq * d:
+        raise KernelError("rope_tied_write: buffers are smaller than the batch")
+    _contig("q_out", q_out), _i32("positions", positions, n)
+    if rot:
+        if cos is None or sin is None or cos.dtype != torch.float32 or sin.dtype != torch.float32 or \
+                cos.shape[1] != rot // 2 or tuple(sin.shape) != tuple(cos.shape):
+            raise KernelError("rope_tied_write: cos and sin are float32 [positions, rot / 2]")
+        _contig("cos", cos), _contig("sin", sin)
+    write = k_cache is not None
+    cache_dt = dtype_code(q_out)
+    if write:
+        if v_cache is None or slots is None:
+            raise KernelError("rope_tied_write: k cache without v cache or slots")
+        _i32("slots", slots, n), _contig("k_cache", k_cache), _contig("v_cache", v_cache)
+        if tuple(k_cache.shape[1:]) != (nkv, page_size, d) or tuple(v_cache.shape) != tuple(k_cache.shape) \
+                or k_cache.dtype != v_cache.dtype:
+            raise KernelError(f"rope_tied_write: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} do not fit "
+                              f"nkv={nkv} page={page_size} d={d}")
+        cache_dt = dtype_code(k_cache)
+    call("pyre_rope_tied_write", proj.data.data_ptr(), dtype_code(proj.data), proj.count, proj.stride, proj.width, col0,
+         _ptr(proj.bias), dtype_code(proj.bias) if proj.bias is not None else 0, q_out.data_ptr(), dtype_code(q_out),
+         _ptr(k_cache), _ptr(v_cache), cache_dt, _ptr(cos) if rot else None, _ptr(sin) if rot else None, int(rot),
+         positions.data_ptr(), _ptr(slots), n, nq, nkv, d, page_size, 1 if write else 0, _stream())
+
+
+def latent_write(proj: Partials, col0: int, q_out: torch.Tensor, c_cache: torch.Tensor | None,
+                 gain: torch.Tensor | None, eps: float, slots: torch.Tensor | None, n: int, q_width: int, rank: int,
+                 page_size: int) -> None:
+    """Finish a step's input product from column ``col0`` on: ``q_width`` columns of queries to ``q_out [N, q_width]``
+    and, if ``c_cache [pages, 1, page, rank]`` is given, the ``rank`` columns behind them divided by their root mean
+    square (``eps`` inside the root), times ``gain``, to the cache at ``slots``."""
+    _dev(proj.data, q_out, c_cache, gain, slots)
+    write = c_cache is not None
+    args = _proj_args(proj, col0, q_width + (rank if write else 0))
+    if proj.rows < n or q_out.numel() < n * q_width:
+        raise KernelError("latent_write: buffers are smaller than the batch")
+    _contig("q_out", q_out)
+    cache_dt = dtype_code(q_out)
+    if write:
+        if gain is None or slots is None or gain.numel() != rank:
+            raise KernelError("latent_write: a cache write needs a gain over the rank and slots")
+        _i32("slots", slots, n), _contig("c_cache", c_cache), _contig("gain", gain)
+        if tuple(c_cache.shape[1:]) != (1, page_size, rank):
+            raise KernelError(f"latent_write: cache {tuple(c_cache.shape)} does not fit page={page_size} rank={rank}")
+        cache_dt = dtype_code(c_cache)
+    call("pyre_latent_write", *args, q_out.data_ptr(), dtype_code(q_out), _ptr(c_cache), cache_dt, _ptr(gain),
+         dtype_code(gain) if gain is not None else 0, float(eps), _ptr(slots), n, q_width, rank, page_size,
+         1 if write else 0, _stream())
+
+
+HEAD_MATMUL_MAX_IN = 1024  #: the widest head that the per-head product takes (latent.hip)
+
+
+def head_matmul(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n: int) -> None:
+    """out[n, h, :] = x[n, h, :] @ w[h] for every head: ``w [heads, din, dout]``, ``x [>= n, heads * din]`` and
+    ``out [>= n, heads * dout]`` with contiguous rows, one element type."""
+    _dev(x, w, out)
+    if w.dim() != 3 or not w.is_contiguous():
+        raise KernelError("head_matmul: w is contiguous [heads, din, dout]")
+    heads, din, dout = w.shape
+    if not (x.dtype == w.dtype == out.dtype):
+        raise KernelError("head_matmul: one element type for x, w and out")
+    if x.dim() != 2 or out.dim() != 2 or x.stride(1) != 1 or out.stride(1) != 1 or x.shape[1] < heads * din or \
+            out.shape[1] < heads * dout or x.shape[0] < n or out.shape[0] < n:
+        raise KernelError("head_matmul: x [>= n, heads*din] and out [>= n, heads*dout] with contiguous rows expected")
+    if din > HEAD_MATMUL_MAX_IN:
+        raise KernelError(f"head_matmul: heads of {din} elements are more than {HEAD_MATMUL_MAX_IN}")
+    call("pyre_head_matmul", x.data_ptr(), x.stride(0), w.data_ptr(), out.data_ptr(), out.stride(0), dtype_code(x), n,
+         heads, din, dout, _stream())
+
+
+ROUTE_MAX_EXPERTS = 512  #: the most experts that the routing kernel chooses among (moe.hip)
+
+
+def route_topk(z: Partials, gates: torch.Tensor, n: int, top: int) -> None:
+    """gates[n, e] (float32 [N, experts]) = s_e / (sum of the chosen s + 1e-20) for the ``top`` experts of largest
+    s = sigmoid(z) (the lower index among equals), 0 for the others; ``z`` the router product's partial sums."""
+    _dev(z.data, z.bias, gates)
+    experts = z.width
+    if gates.dtype != torch.float32 or not gates.is_contiguous() or gates.dim() != 2 or gates.shape[1] != experts or \
+            gates.shape[0] < n or z.rows < n:
+        raise KernelError("route_topk: gates are contiguous float32 [>= n, experts]")
+    if not (0 < top <= experts <= ROUTE_MAX_EXPERTS):
+        raise KernelError(f"route_topk: {top} of {experts} experts is not a choice this kernel makes")
+    call("pyre_route_topk", *z._args(experts), gates.data_ptr(), n, experts, int(top), _stream())
+
+
+def expert_act(up: Partials, gates: torch.Tensor, out: torch.Tensor, n: int, experts: int, ff: int, shared_ff: int) -> None:
+    """out[n, e*ff + j] = gates[n, e] * relu(up[n, e*ff + j])^2 for the routed experts, relu(up)^2 for the
+    ``shared_ff`` columns behind them; ``up`` the partial sums of the product over all experts' matrices."""
+    _dev(up.data, gates, out)
+    width = experts * ff + shared_ff
+    if up.bias is not None:
+        raise KernelError("expert_act: a pending bias is not supported")
+    if up.width != width or up.rows < n or out.shape[-1] != width or out.shape[0] < n:
+        raise KernelError("expert_act: the product's width does not fit experts * ff + shared_ff")
+    if gates.dtype != torch.float32 or not gates.is_contiguous() or gates.shape[-1] != experts or gates.shape[0] < n:
+        raise KernelError("expert_act: gates are contiguous float32 [>= n, experts]")
+    _contig("out", out)
+    call("pyre_expert_act", up.data.data_ptr(), dtype_code(up.data), up.count, up.stride, gates.data_ptr(),
+         out.data_ptr(), dtype_code(out), n, experts, ff, shared_ff, _stream())

@@ -295,6 +295,9 @@ class RotarySpec:
     theta: float
     max_positions: int
     rotary_dim: int | None = None    #: None: the whole head
+    #: angles position * theta^(-2j/d) formed in float64 and their cosines and sines rounded to float32 once,
+    #: instead of float32 arithmetic all the way
+    exact: bool = False
     kind: ClassVar[str] = "rotary"
 
 
@@ -375,6 +378,93 @@ class GatedLinearAttentionSpec:
 
 
 @dataclass(frozen=True)
+class TanhNormSpec:
+    """tanh(alpha x) * gain + shift, element by element: a norm that takes no statistic of the row. ``name`` is
+    the gain's tensor; the scalar and the shift are ``name + ".alpha"`` and ``name + ".b"``."""
+
+    hidden_size: int
+    name: str
+    kind: ClassVar[str] = "tanh_norm"
+
+
+@dataclass(frozen=True)
+class TiedAttentionSpec:
+    """Grouped softmax attention whose values are its keys as projected (before any rotation): there is no value
+    matrix. Scores times ``scale``; ``chunk`` = C > 0 lets a query see only the earlier keys of its own run of C
+    positions (runs counted from position 0), 0 is plain causal attention. ``position`` describes the rotation of
+    queries and keys (or none). Tensors: ``prefix + .q / .k / .o`` and, with ``bias``, ``.q.b / .k.b``."""
+
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    head_dim: int
+    scale: float
+    position: Any
+    prefix: str
+    chunk: int = 0
+    bias: bool = True
+    kind: ClassVar[str] = "tied_attention"
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Causal softmax attention whose keys and values of all heads are made of one compressed row per token:
+    c = rms_norm(Wdkv h) * gain [rank]; per head k = Wuk c (``key_dim``), v = Wuv c (``value_dim``). Only c is
+    kept. ``own_latent`` False: the layer has no Wdkv and reads the rows that another layer keeps (the order of
+    layers names it as the entry whose cache this one reads). Tensors: ``prefix + .q / .dkv / .dkv.norm / .uk /
+    .uv / .o``."""
+
+    hidden_size: int
+    num_heads: int
+    key_dim: int
+    value_dim: int
+    rank: int
+    scale: float
+    norm_eps: float
+    prefix: str
+    own_latent: bool = True
+    kind: ClassVar[str] = "latent_attention"
+
+
+@dataclass(frozen=True)
+class GeluGLUSpec:
+    """down(gelu_tanh(gate(x)) * up(x)), no biases. Tensors: ``prefix + .gate / .up / .down``."""
+
+    hidden_size: int
+    intermediate_size: int
+    prefix: str
+    kind: ClassVar[str] = "gelu_glu"
+
+
+@dataclass(frozen=True)
+class SigmoidMoESpec:
+    """A mixture of ``experts`` feed-forward layers down(relu(up(x))^2) of ``expert_size`` hidden units each: every
+    token goes through the ``top`` experts of largest sigmoid(router(x)), weighted by these scores over their sum
+    (+ 1e-20); a shared expert of ``shared_size`` units (0: none) runs for every token and is added. Tensors:
+    ``prefix + .router``, ``.e<i>.up / .down``, ``.shared.up / .down``."""
+
+    hidden_size: int
+    experts: int
+    top: int
+    expert_size: int
+    prefix: str
+    shared_size: int = 0
+    kind: ClassVar[str] = "sigmoid_moe"
+
+
+@dataclass(frozen=True)
+class ParallelBlockSpec:
+    """x += scale * (mixer(norm(x)) + feed_forward(norm(x))): one norm, both sublayers read its rows
+    (``feed_forward`` None: the mixer alone)."""
+
+    mixer: Any
+    norm: Any
+    feed_forward: Any = None
+    scale: float = 1.0
+    kind: ClassVar[str] = "parallel_block"
+
+
+@dataclass(frozen=True)
 class ParallelMixerSpec:
     """sum_i scales[i] * branches[i](h): mixers side by side that read the same rows."""
 
@@ -449,6 +539,7 @@ class LMHeadSpec:
     name: str = "lm_head.weight"
     tied_to: str | None = None       #: embedding tensor used when the head is tied
     scale: float = 1.0               #: the logits are multiplied by this
+    softcap: float = 0.0             #: c > 0: then squashed, c * tanh(logit / c)
     kind: ClassVar[str] = "lm_head"
 
 

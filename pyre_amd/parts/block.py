@@ -7,7 +7,7 @@ from dataclasses import dataclass
 import torch
 
 from pyre_amd.hip.ops import Partials, PostNorm
-from pyre_amd.parts.base import Block, BlockSpec, SandwichBlockSpec, TensorSpec, make_part, take
+from pyre_amd.parts.base import Block, BlockSpec, ParallelBlockSpec, SandwichBlockSpec, TensorSpec, make_part, take
 
 
 @dataclass
@@ -126,3 +126,47 @@ class SandwichBlock(Block):
         self.feed_forward_norm.forward(ctx, state.resid, state.pending, h)
         state.pending = self._post(self.feed_forward.forward(ctx, h), self.feed_forward_post,
                                    self.spec.feed_forward_scale)
+
+
+class ParallelBlock(Block):
+    """x += scale * (mixer(norm(x)) + feed_forward(norm(x))): one norm whose rows both sublayers read. Neither
+    result is added here: both are handed on as the pending term (the second as ``Partials.more``, each with the
+    factor), and the next norm's kernel adds them to the residual stream as it norms."""
+
+    def __init__(self, spec: ParallelBlockSpec):
+        self.spec = spec
+        self.norm = make_part("norm", spec.norm)
+        self.mixer = make_part("mixer", spec.mixer)
+        self.feed_forward = make_part("feed_forward", spec.feed_forward) if spec.feed_forward is not None else None
+
+    def parts(self):
+        return tuple(p for p in (self.norm, self.mixer, self.feed_forward) if p is not None)
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return [s for p in self.parts() for s in p.tensor_specs()]
+
+    def bind(self, tensors, runtime) -> None:
+        for p in self.parts():
+            p.bind(tensors, runtime)
+
+    def linears(self) -> list:
+        return [lin for p in self.parts() for lin in p.linears()]
+
+    def cache_specs(self) -> list:
+        spec = self.mixer.cache_spec()
+        return [] if spec is None else [spec]
+
+    def step_arrays(self) -> list:
+        return self.mixer.step_arrays()
+
+    def forward(self, ctx, state: Hidden, caches: list) -> None:
+        h = ctx.workspace.get("block.h", (ctx.n_tokens, state.resid.shape[1]), ctx.dtype)
+        self.norm.forward(ctx, state.resid, state.pending, h)
+        mixed = self.mixer.forward(ctx, h, caches[0] if caches else None)
+        if mixed.post is not None or mixed.more is not None or mixed.scale != 1.0:
+            raise ValueError("a parallel block takes a sublayer's plain result")
+        more = None
+        if self.feed_forward is not None:
+            fed = self.feed_forward.forward(ctx, h)
+            more = Partials(fed.data, fed.bias, scale=self.spec.scale)
+        state.pending = Partials(mixed.data, mixed.bias, scale=self.spec.scale, more=more)

@@ -2,14 +2,17 @@
 
 from pyre_amd.parts.attention import Attention
 from pyre_amd.parts.base import register_part
-from pyre_amd.parts.block import PreNormBlock, SandwichBlock
+from pyre_amd.parts.block import ParallelBlock, PreNormBlock, SandwichBlock
 from pyre_amd.parts.branch import ParallelMixer
 from pyre_amd.parts.capped_attention import CappedAttention
 from pyre_amd.parts.embedding import LMHead, TokenEmbedding
-from pyre_amd.parts.feedforward import ClippedGLU, SwiGLU
+from pyre_amd.parts.feedforward import ClippedGLU, GeluGLU, SwiGLU
+from pyre_amd.parts.latent_attention import LatentAttention
 from pyre_amd.parts.linear_attention import GatedLinearAttention
-from pyre_amd.parts.norm import LayerNorm, RMSNorm
+from pyre_amd.parts.moe import SigmoidMoE
+from pyre_amd.parts.norm import LayerNorm, RMSNorm, TanhNorm
 from pyre_amd.parts.rotary import NoPosition, RotaryEncoding
+from pyre_amd.parts.tied_attention import TiedAttention
 
 register_part("mixer", "attention", Attention)
 register_part("feed_forward", "swiglu", SwiGLU)
@@ -25,3 +28,9 @@ register_part("mixer", "parallel", ParallelMixer)
 register_part("feed_forward", "clipped_glu", ClippedGLU)
 register_part("norm", "layernorm", LayerNorm)
 register_part("block", "sandwich", SandwichBlock)
+register_part("mixer", "tied_attention", TiedAttention)
+register_part("mixer", "latent_attention", LatentAttention)
+register_part("feed_forward", "gelu_glu", GeluGLU)
+register_part("feed_forward", "sigmoid_moe", SigmoidMoE)
+register_part("norm", "tanh_norm", TanhNorm)
+register_part("block", "parallel_block", ParallelBlock)

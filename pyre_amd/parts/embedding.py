@@ -50,4 +50,6 @@ class LMHead(Part):
             ops.reduce_partials(p, out, m)
         if self.spec.scale != 1.0:
             ops.scale_(out, self.spec.scale)
+        if self.spec.softcap:
+            ops.softcap_(out, self.spec.softcap)
         return out

@@ -90,7 +90,8 @@ def mid_ksplit(n_out: int, k: int, block_rows: int = 64, units: int = DEFAULT_UN
 # gated unit with clipped inputs (measured on a four-layer model of 512 columns: whole prompts 0.059 -> the
 # 0.026 of short portions, whose products hand on float32 partial sums anyway).
 LIBRARY_F32_ROLES = frozenset({"attn.qkv", "attn.out", "mix.in", "mix.out", "cattn.in", "cattn.out", "gla.in", "gla.out",
-                               "glu.down"})
+                               "glu.down", "tattn.qk", "tattn.out", "lattn.in", "lattn.out", "geglu.down", "moe.router",
+                               "moe.down"})
 
 
 def _is_bf16(ctx, lin, x) -> bool:

@@ -6,7 +6,7 @@ import torch
 
 from pyre_amd.hip import ops
 from pyre_amd.parts import fast
-from pyre_amd.parts.base import ClippedGLUSpec, FeedForward, SwiGLUSpec, TensorSpec, take
+from pyre_amd.parts.base import ClippedGLUSpec, FeedForward, GeluGLUSpec, SwiGLUSpec, TensorSpec, take
 from pyre_amd.parts.linear import Linear, linear_specs
 
 
@@ -78,4 +78,43 @@ class ClippedGLU(FeedForward):
         if not fast.gate_up_silu(self.gate_up, ctx, h, n, act, unit=(self.spec.limit, self.spec.slope, 1.0)):
             gu = self.gate_up.forward(ctx, h, n)
             ops.clipped_glu(gu, act, n, self.spec.limit, self.spec.slope)
+        return self.down.forward(ctx, act, n)
+
+
+class GeluGLU(FeedForward):
+    """down(gelu_tanh(gate(x)) * up(x)): the gated unit g sigmoid(slope (g + cubic g^3)) u, which is the tanh form of
+    GELU on the gate since (1 + tanh z) / 2 = sigmoid(2 z). gate and up are one product over [Wgate; Wup]; a step of
+    few rows finishes the unit in that product's epilogue."""
+
+    UNIT = (0.0, ops.GELU_TANH_SLOPE, 0.0, ops.GELU_TANH_CUBIC)  #: no clipping, no shift
+
+    def __init__(self, spec: GeluGLUSpec):
+        self.spec = spec
+        self.gate_up = Linear(spec.hidden_size, 2 * spec.intermediate_size, "ffn.gate_up")
+        self.down = Linear(spec.intermediate_size, spec.hidden_size, "geglu.down")
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        s, p = self.spec, self.spec.prefix
+        return [TensorSpec(f"{p}.gate", (s.intermediate_size, s.hidden_size)),
+                TensorSpec(f"{p}.up", (s.intermediate_size, s.hidden_size)),
+                TensorSpec(f"{p}.down", (s.hidden_size, s.intermediate_size))]
+
+    def bind(self, tensors, runtime) -> None:
+        p = self.spec.prefix
+        halves = [take(tensors, f"{p}.gate"), take(tensors, f"{p}.up")]
+        fused = torch.cat(halves, dim=0)
+        del halves
+        self.gate_up.set(fused)
+        self.down.set(take(tensors, f"{p}.down"))
+
+    def linears(self) -> list:
+        return [self.gate_up, self.down]
+
+    def forward(self, ctx, h):
+        n = ctx.n_tokens
+        act = ctx.workspace.get("ffn.act", (n, self.spec.intermediate_size), ctx.dtype)
+        if not fast.gate_up_silu(self.gate_up, ctx, h, n, act, unit=self.UNIT):
+            gu = self.gate_up.forward(ctx, h, n)
+            limit, slope, shift, cubic = self.UNIT
+            ops.clipped_glu(gu, act, n, limit, slope, shift, cubic)
         return self.down.forward(ctx, act, n)

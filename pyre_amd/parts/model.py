@@ -108,7 +108,7 @@ class LayeredModel(Part):
         included (its partial sums in their order, then the bias)."""
         rows = state.resid[:ctx.n_tokens].clone()
         p = state.pending
-        if p is not None:
+        while p is not None:
             term = torch.zeros_like(rows)
             for i in range(p.count):
                 term += p.data[i, :ctx.n_tokens].float()
@@ -119,5 +119,6 @@ class LayeredModel(Part):
                 term = dev / torch.sqrt((dev * dev).mean(-1, keepdim=True) + p.post.eps) * p.post.gain.float()
                 if p.post.scale is not None:
                     term = term * p.post.scale.float()
-            rows += term
+            rows += term * p.scale
+            p = p.more
         return rows

@@ -3,7 +3,7 @@
 from __future__ import annotations
 
 from pyre_amd.hip import ops
-from pyre_amd.parts.base import LayerNormSpec, Norm, RMSNormSpec, TensorSpec
+from pyre_amd.parts.base import LayerNormSpec, Norm, RMSNormSpec, TanhNormSpec, TensorSpec, take
 
 
 class RMSNorm(Norm):
@@ -38,3 +38,28 @@ class LayerNorm(Norm):
 
     def forward(self, ctx, resid, delta, out, rows=None) -> None:
         ops.add_layernorm(resid, delta, self.gain, self.spec.eps, out, rows)
+
+
+class TanhNorm(Norm):
+    """tanh(alpha x) * gain + shift with one learned number alpha: no mean, no variance, so a row is normed
+    element by element. Fused with the residual sum before it; takes up to two pending terms, each with a factor
+    (``Partials.scale``, ``Partials.more``)."""
+
+    def __init__(self, spec: TanhNormSpec):
+        self.spec = spec
+        self.gain = self.shift = self.alpha = None
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        n, h = self.spec.name, self.spec.hidden_size
+        # random weights: alpha one, so that rows of unit scale use the bend of the tanh
+        return [TensorSpec(n, (h,), init="gain"), TensorSpec(f"{n}.b", (h,), init="normal"),
+                TensorSpec(f"{n}.alpha", (), init="gain")]
+
+    def bind(self, tensors, runtime) -> None:
+        n = self.spec.name
+        self.gain = take(tensors, n).contiguous()
+        self.shift = take(tensors, f"{n}.b").to(self.gain.dtype).contiguous()
+        self.alpha = take(tensors, f"{n}.alpha").to(self.gain.dtype).reshape(1).contiguous()
+
+    def forward(self, ctx, resid, delta, out, rows=None) -> None:
+        ops.add_tanhnorm(resid, delta, self.alpha, self.gain, self.shift, out, rows)

@@ -14,8 +14,13 @@ import torch
 from pyre_amd.parts.base import NoPositionSpec, PositionEncoding, RotarySpec
 
 
-def rotary_tables(rotary_dim: int, theta: float, n_positions: int) -> tuple[torch.Tensor, torch.Tensor]:
-    """cos, sin of shape [n_positions, rotary_dim / 2], float32, on the CPU."""
+def rotary_tables(rotary_dim: int, theta: float, n_positions: int, exact: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
+    """cos, sin of shape [n_positions, rotary_dim / 2], float32, on the CPU. ``exact``: the angles are formed in
+    float64 and only their cosines and sines are rounded."""
+    if exact:
+        inv = theta ** (-torch.arange(0, rotary_dim, 2, dtype=torch.float64) / rotary_dim)
+        freqs = torch.outer(torch.arange(n_positions, dtype=torch.float64), inv)
+        return freqs.cos().float(), freqs.sin().float()
     inv_freq = 1.0 / (theta ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
     t = torch.arange(n_positions, dtype=torch.float32)
     freqs = torch.outer(t, inv_freq)
@@ -33,7 +38,7 @@ class RotaryEncoding(PositionEncoding):
     def rotary(self, runtime):
         n = runtime.max_positions  # the engine's longest request decides, as the reference's table grows on demand
         if self._tables is None or self._tables[0].shape[0] < n or self._tables[0].device != runtime.device:
-            cos, sin = rotary_tables(self.rotary_dim, self.spec.theta, n)
+            cos, sin = rotary_tables(self.rotary_dim, self.spec.theta, n, self.spec.exact)
             self._tables = (cos.to(runtime.device).contiguous(), sin.to(runtime.device).contiguous())
         return self._tables[0], self._tables[1], self.rotary_dim
 
