@@ -186,3 +186,29 @@ def forward(w, cfg, ids, return_hidden=False):
     if cap:
         z = cap * torch.tanh(z / cap)
     return (z, hidden) if return_hidden else z
+
+
+def closest_call(w, cfg, ids):
+    """Per position the smallest gap, over the layers with a mixture, between the scores of the last expert that is
+    chosen and the first that is not (infinite where nothing is left out): where it is tiny, rounding decides which
+    experts a token goes through, and its row is no measure of an engine in 16 bits."""
+    x = w["embed"][torch.as_tensor(ids, dtype=torch.long)].clone()
+    eps, mult = cfg["norm"]["eps"], cfg["residual_mult"]
+    latents, gap = {}, torch.full((len(ids),), float("inf"), dtype=F)
+    for i, layer in enumerate(cfg["layers"]):
+        p, m, mlp = f"l{i}", layer["mixer"], layer.get("mlp")
+        h = squash_norm(x, w, p + ".norm1")
+        if layer["type"] == "attention":
+            y = chunked_attention(h, w, p + ".mix", m)
+        else:
+            src = m.get("kv_from")
+            latents[i] = latents[src] if src is not None else latent_of(h, w, p + ".mix", eps)
+            y = latent_attention(h, latents[i], w, p + ".mix", m)
+        if mlp is not None:
+            if mlp["kind"] == "moe" and mlp["router"]["top"] < mlp["router"]["experts"]:
+                s = torch.sigmoid(h @ w[p + ".mlp.router"].T).sort(dim=-1, descending=True).values
+                top = mlp["router"]["top"]
+                gap = torch.minimum(gap, s[:, top - 1] - s[:, top])
+            y = y + feed_forward(h, w, p + ".mlp", mlp)
+        x = x + mult * y
+    return gap
