@@ -12,6 +12,7 @@
 // All arithmetic is float32.
 #include "pyre_api.h"
 #include "pyre_common.h"
+#include "pyre_vec4.h"
 
 using namespace pyre;
 
@@ -80,6 +81,27 @@ __global__ __launch_bounds__(256) void expert_act_kernel(const void* __restrict_
   store_from_float(out, out_dt, i, y);
 }
 
+// Four columns a thread (the experts' sizes, the shared expert's and the partial sums' stride are multiples of four,
+// so the four share an expert); columns of an expert that the token does not take are not read.
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void expert_act_vec_kernel(const TI* __restrict__ up, int n_partials, size_t partial_stride,
+                                                             const float* __restrict__ gates, TO* __restrict__ out,
+                                                             size_t total4, int experts, int ff, int width) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= total4) return;
+  const int per_row = width / 4;
+  const size_t n = i / per_row;
+  const int c = 4 * static_cast<int>(i % per_row), e = c / ff;
+  const float g = e < experts ? gates[n * experts + e] : 1.f;
+  float4 y = {0.f, 0.f, 0.f, 0.f};
+  if (g != 0.f) {
+    const float4 u = sum_partials4(up + n * width + c, partial_stride, n_partials);
+    const float a = fmaxf(u.x, 0.f), b = fmaxf(u.y, 0.f), cc = fmaxf(u.z, 0.f), d = fmaxf(u.w, 0.f);
+    y = float4{g * (a * a), g * (b * b), g * (cc * cc), g * (d * d)};
+  }
+  Vec4<TO>::store(out + n * width + c, y);
+}
+
 }  // namespace
 
 extern "C" int pyre_route_topk(const void* z, int z_dt, int n_partials, long partial_stride, const void* bias, int bias_dt,
@@ -100,6 +122,14 @@ extern "C" int pyre_expert_act(const void* up, int up_dt, int n_partials, long p
   if (n <= 0) return 0;
   const int width = experts * ff + shared_ff;
   const size_t total = static_cast<size_t>(n) * width;
+  if (ff % 4 == 0 && shared_ff % 4 == 0 && partial_stride % 4 == 0 && reinterpret_cast<uintptr_t>(up) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+    PYRE_DISPATCH(up_dt, TI, PYRE_DISPATCH(out_dt, TO,
+        hipLaunchKernelGGL((expert_act_vec_kernel<TI, TO>), dim3((total / 4 + 255) / 256), dim3(256), 0, stream,
+                           static_cast<const TI*>(up), n_partials, static_cast<size_t>(partial_stride), gates,
+                           static_cast<TO*>(out), total / 4, experts, ff, width)));
+    return check_launch("expert_act");
+  }
   hipLaunchKernelGGL(expert_act_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, up, up_dt, n_partials,
                      static_cast<size_t>(partial_stride), gates, out, out_dt, total, experts, ff, width);
   return check_launch("expert_act");

@@ -1070,7 +1070,7 @@ def latent_write(proj: Partials, col0: int, q_out: torch.Tensor, c_cache: torch.
          1 if write else 0, _stream())
 
 
-HEAD_MATMUL_MAX_IN = 1024  #: the widest head that the per-head product takes (latent.hip)
+HEAD_MATMUL_MAX_IN = 768  #: the widest head that the per-head product takes (latent.hip)
 
 
 def head_matmul(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n: int) -> None:
