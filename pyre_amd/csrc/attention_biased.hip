@@ -18,7 +18,8 @@
 // attn_biased_tile    prompt portions: tiles of up to 32 consecutive tokens of a request, four query
 //                 heads of a key/value head per block, chunks of 32 keys through LDS, both products on
 //                 the matrix cores' float32 instruction (scores and weights stay float32).
-// attn_biased_single  single tokens: a block per (token, query head), the keys in spans of 128.
+// attn_biased_single  single tokens: a block per (token, up to eight query heads of a key/value head), the keys in
+//                 spans of 128 that the block's heads read together.
 //
 // Chunks start at multiples of 32 keys and spans at the token's first visible key, so the order of
 // every sum of a token depends on its own bounds alone.
@@ -384,114 +385,361 @@ __global__ __launch_bounds__(kThreads) void attn_biased_tile_kernel(
     }
 }
 
+// The tile kernel for bfloat16 queries and caches, on the matrix cores' 16-bit instruction with nothing rounded that
+// the float32 form keeps: a product of two bfloat16 values is exact in float32, so S^T = K Q^T is what the float32
+// instruction gives (sums in float32 either way); and a float32 weight p is split into three bfloat16 pieces
+// p = p1 + p2 + p3 (p1 = bf16(p), p2 = bf16(p - p1), p3 = p - p1 - p2, which has eight bits left: exact), each
+// multiplied with the values and added in float32: scores and weights stay 32-bit. 32 such instructions a chunk and
+// head of 128 where the float32 form has 128, keys, queries and values as bfloat16 in LDS (a third of the space, so
+// that three blocks share a compute unit). Head sizes are multiples of eight; the caches start on 16 bytes.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+constexpr int kPad16 = 8;            // bfloat16 elements of padding behind a row of keys, queries or transposed values
+
+// Where key kk of a chunk lies in a row of transposed values: the eight keys that a lane multiplies in one
+// instruction (kk = 16 a + 4 h + u and 16 a + 8 + 4 h + u, u < 4) side by side, one 16-byte read.
+__device__ inline int vt_slot(int kk) { return (kk & 16) + 8 * ((kk >> 2) & 1) + 4 * ((kk >> 3) & 1) + (kk & 3); }
+
+template <int NV>
+__global__ __launch_bounds__(kThreads) void attn_biased_tile16_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, bf16* __restrict__ out,
+    int out_ld, const float* __restrict__ gate, float out_scale, const int* __restrict__ tiles,
+    const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
+    int table_stride, int nq, int nkv, int dk, int dkp, int dv, int page_size, float scale, float cap,
+    const float* __restrict__ bias, int far, int window, int keep_first, int chunk, int tab_lds, int bias_lds) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const int ldk = dkp + kPad16, ldv = kKeys + kPad16;
+  bf16* Ks = reinterpret_cast<bf16*>(lds_raw);                 // [kKeys][ldk]
+  bf16* Qs = Ks + kKeys * ldk;                                 // [4 waves][32 tokens][ldk]
+  bf16* Vt = Qs + 4 * 32 * ldk;                                // [32 NV][ldv], keys in the order of vt_slot
+  int* tab_s = reinterpret_cast<int*>(Vt + 32 * NV * ldv);     // [tab_lds]: the request's block table, if it fits
+  float* bias_s = reinterpret_cast<float*>(tab_s + tab_lds);   // [4][far + 1]: the four heads' biases, if they fit
+  __shared__ int page_s[2][kKeys];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, h = lane >> 5, c = lane & 31;
+  const int n_rep = nq / nkv, hgroups = (n_rep + 3) / 4;
+  const int kvh = blockIdx.y / hgroups, hin = (blockIdx.y % hgroups) * 4 + wave;
+  const bool active = hin < n_rep;  // a wave without a head still helps loading
+  const int head = kvh * n_rep + (active ? hin : 0);
+  const int t0 = tiles[2 * blockIdx.x], ntok = tiles[2 * blockIdx.x + 1];
+  if (ntok <= 0) return;
+  const int pos0 = positions[t0];
+  const int* table = block_table + static_cast<size_t>(seq_of_token[t0]) * table_stride;
+
+  const bool live = active && c < ntok;
+  const int hi = c < ntok ? pos0 + c : pos0;
+  const int lo = first_seen(hi, window, chunk);
+  const int keep = window > 0 ? keep_first : 0;
+  const float* bias_row = bias ? bias + static_cast<size_t>(head) * (far + 1) : nullptr;
+  for (int i = tid; i < tab_lds; i += kThreads) tab_s[i] = table[i];
+  if (bias && bias_lds) {
+    for (int i = lane; i <= far; i += 64) bias_s[wave * (far + 1) + i] = bias_row[i];
+    bias_row = bias_s + wave * (far + 1);
+  }
+  const uint4 zero4 = {0u, 0u, 0u, 0u};
+  {  // this wave's queries: Qs[wave][token][d], zeros where there is no token or no element
+    bf16* mine = Qs + wave * 32 * ldk;
+    for (int i = lane; i < 32 * (dkp / 8); i += 64) {
+      const int t = i / (dkp / 8), d = 8 * (i % (dkp / 8));
+      uint4 v = zero4;
+      if (active && t < ntok && d < dk) v = *reinterpret_cast<const uint4*>(q + (static_cast<size_t>(t0 + t) * nq + head) * dk + d);
+      *reinterpret_cast<uint4*>(mine + t * ldk + d) = v;
+    }
+  }
+  const bf16* myq = Qs + wave * 32 * ldk + c * ldk + 8 * h;
+  f32x16 o[NV];
+#pragma unroll
+  for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[dt][i] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  const int lo_all = first_seen(pos0, window, chunk);
+  const int hi_all = pos0 + ntok - 1;
+  const int kept_end = min(keep, lo_all);
+  const int n_first = kept_end > 0 ? (kept_end - 1) / kKeys + 1 : 0;
+  const int chunk_b = max(lo_all / kKeys, n_first);
+  const int n_chunks = n_first + (hi_all / kKeys - chunk_b + 1);
+  // the next chunk's keys and values are asked for (into registers) before the current chunk is multiplied, and go
+  // to LDS when every wave is done with it
+  constexpr int KI = kKeys * (kTileMaxKeyHead / 8) / kThreads, VI = (kKeys * 4 * NV + kThreads - 1) / kThreads;
+  uint4 kreg[KI], vreg[VI];
+  auto chunk_key0 = [&](int it) { return (it < n_first ? it : chunk_b + (it - n_first)) * kKeys; };
+  auto page_of = [&](int key) {
+    const int entry = key / page_size;
+    if (key > hi_all || entry >= table_stride) return -1;
+    return entry < tab_lds ? tab_s[entry] : table[entry];
+  };
+  auto ask = [&](int it) {
+    const int key0 = chunk_key0(it), kg = dkp / 8;
+    if (tid < kKeys) page_s[it & 1][tid] = page_of(key0 + tid);
+#pragma unroll
+    for (int k = 0; k < KI; ++k) {
+      const int i = tid + k * kThreads, key = key0 + i / kg, d = 8 * (i % kg);
+      const int page = i < kKeys * kg ? page_of(key) : -1;
+      kreg[k] = zero4;
+      if (page >= 0 && d < dk)
+        kreg[k] = *reinterpret_cast<const uint4*>(k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + key % page_size) * dk + d);
+    }
+#pragma unroll
+    for (int k = 0; k < VI; ++k) {
+      const int i = tid + k * kThreads, key = key0 + i / (4 * NV), d = 8 * (i % (4 * NV));
+      const int page = i < kKeys * 4 * NV ? page_of(key) : -1;
+      vreg[k] = zero4;
+      if (page >= 0 && d < dv)
+        vreg[k] = *reinterpret_cast<const uint4*>(v_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + key % page_size) * dv + d);
+    }
+  };
+  auto stash = [&]() {
+    const int kg = dkp / 8;
+#pragma unroll
+    for (int k = 0; k < KI; ++k) {
+      const int i = tid + k * kThreads, key = i / kg, d = 8 * (i % kg);
+      if (i < kKeys * kg) *reinterpret_cast<uint4*>(Ks + key * ldk + d) = kreg[k];
+    }
+#pragma unroll
+    for (int k = 0; k < VI; ++k) {
+      const int i = tid + k * kThreads, key = i / (4 * NV), d = 8 * (i % (4 * NV));
+      if (i < kKeys * 4 * NV) {
+        const uint32_t w[4] = {vreg[k].x, vreg[k].y, vreg[k].z, vreg[k].w};
+        const int slot = vt_slot(key);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) Vt[(d + u) * ldv + slot].bits = static_cast<uint16_t>(u & 1 ? w[u >> 1] >> 16 : w[u >> 1] & 0xffffu);
+      }
+    }
+  };
+  __syncthreads();  // the table and the biases are in LDS
+  ask(0);
+  for (int it = 0; it < n_chunks; ++it) {
+    const int key0 = chunk_key0(it);
+    const int* pages = page_s[it & 1];
+    __syncthreads();  // the previous chunk has been read by every wave (and the queries are written)
+    stash();
+    __syncthreads();
+    if (it + 1 < n_chunks) ask(it + 1);
+    if (!active) continue;
+
+    f32x16 s;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+    const bf16* krow = Ks + c * ldk + 8 * h;
+#pragma unroll 4
+    for (int st = 0; st < dkp; st += 16) {  // elements st + 8 h .. st + 8 h + 7 of the key and the query
+      const bf16x8 k8 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(krow + st));
+      const bf16x8 q8 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(myq + st));
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k8, q8, s, 0, 0, 0);
+    }
+
+    // element i of s: key key0 + 8 (i / 4) + 4 h + i % 4, token c
+    float bv[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int key = key0 + 8 * (i >> 2) + 4 * h + (i & 3);
+      bv[i] = bias_row ? bias_row[min(max(hi - key, 0), far)] : 0.f;
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int kk = 8 * (i >> 2) + 4 * h + (i & 3), key = key0 + kk;
+      const bool seen = key <= hi && (key >= lo || key < keep) && pages[kk] >= 0;
+      const float shaped = shaped_score(s[i], scale, cap, nullptr, 0, 0) + bv[i];
+      s[i] = seen ? shaped : -INFINITY;
+      mx = fmaxf(mx, s[i]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = expf(m - m_use);
+    m = m_new;
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      s[i] = expf(s[i] - m_use);
+      sum += s[i];
+    }
+    l = l * alpha + sum;
+#pragma unroll
+    for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+    // the weights in three bfloat16 pieces each; piece[a]: the lane's eight keys of instruction a (s[8 a .. 8 a + 7])
+    uint4 piece[3][2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      uint32_t w1[4], w2[4], w3[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float p0 = s[8 * a + 2 * u], p1 = s[8 * a + 2 * u + 1];
+        w1[u] = pack_bf16x2(p0, p1);
+        const float r0 = p0 - __uint_as_float(w1[u] << 16), r1 = p1 - __uint_as_float(w1[u] & 0xffff0000u);
+        w2[u] = pack_bf16x2(r0, r1);
+        w3[u] = pack_bf16x2(r0 - __uint_as_float(w2[u] << 16), r1 - __uint_as_float(w2[u] & 0xffff0000u));
+      }
+      piece[0][a] = uint4{w1[0], w1[1], w1[2], w1[3]};
+      piece[1][a] = uint4{w2[0], w2[1], w2[2], w2[3]};
+      piece[2][a] = uint4{w3[0], w3[1], w3[2], w3[3]};
+    }
+#pragma unroll
+    for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+      for (int a = 0; a < 2; ++a) {
+        const bf16x8 v8 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(Vt + (32 * dt + c) * ldv + 16 * a + 8 * h));
+#pragma unroll
+        for (int pc = 2; pc >= 0; --pc)  // the smallest pieces first
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v8, __builtin_bit_cast(bf16x8, piece[pc][a]), o[dt], 0, 0, 0);
+      }
+  }
+
+  if (!active) return;
+  l += __shfl_xor(l, 32, 64);
+  if (!live) return;
+  float f = (l > 0.f ? 1.f / l : 0.f) * out_scale;
+  if (gate) f *= gate[static_cast<size_t>(t0 + c) * nq + head];
+  bf16* dst = out + static_cast<size_t>(t0 + c) * out_ld + head * dv;
+#pragma unroll
+  for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int d = 32 * dt + 8 * (i >> 2) + 4 * h + (i & 3);
+      if (d < dv) dst[d] = from_float<bf16>(o[dt][i] * f);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 constexpr int kSpan = 128;
 constexpr int kMaxHead = 256;
 
-// VEC: the key head is a multiple of eight elements and the cache starts on 16 bytes (a key in 16-byte loads).
+// A block: one token, up to kGroup query heads of one key/value head, the keys in spans of 128. The heads share what
+// the block reads: a thread takes a key's row once for its heads' scores (two threads a key, each with every second
+// head), and a value once for all heads' sums. VEC: the key head is a multiple of eight elements and the cache starts
+// on 16 bytes (a key in 16-byte loads).
+constexpr int kGroup = 8;
 template <typename T, bool VEC>
 __global__ __launch_bounds__(kThreads) void attn_biased_single_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, T* __restrict__ out,
     int out_ld, const float* __restrict__ gate, float out_scale, const int* __restrict__ tokens,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, int nq, int nkv, int dk, int dv, int page_size, float scale, float cap,
-    const float* __restrict__ bias, int far, int window, int keep_first, int chunk, float* __restrict__ part) {
-  __shared__ __attribute__((aligned(16))) float qs[kMaxHead];
-  __shared__ float sc[kSpan];
+    const float* __restrict__ bias, int far, int window, int keep_first, int chunk, int hg, float* __restrict__ part) {
+  __shared__ __attribute__((aligned(16))) float qs[kGroup][kMaxHead];
+  __shared__ float sc[kGroup][kSpan];
   __shared__ int row_s[kSpan];
-  __shared__ float accs[kThreads];
-  __shared__ float scratch[16];
-  const int n = tokens ? tokens[blockIdx.x] : blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
-  const int kvh = h / (nq / nkv);
+  __shared__ float accs[kGroup][kThreads];
+  __shared__ float m_s[kGroup], l_s[kGroup], alpha_s[kGroup];
+  const int n = tokens ? tokens[blockIdx.x] : blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int rep = nq / nkv, hgroups = (rep + hg - 1) / hg;
+  const int kvh = blockIdx.y / hgroups, first = (blockIdx.y % hgroups) * hg, nh = min(hg, rep - first);
+  const int h0 = kvh * rep + first;  // the block's heads are h0 .. h0 + nh - 1
   const int pos = positions[n];
   const int* table = block_table + static_cast<size_t>(seq_of_token[n]) * table_stride;
   const int lo = first_seen(pos, window, chunk);
   const int kept_end = window > 0 ? min(keep_first, lo) : 0;  // keys 0 .. kept_end - 1, then lo .. pos
-  const float* bias_row = bias ? bias + static_cast<size_t>(h) * (far + 1) : nullptr;
   const int spans_first = (kept_end + kSpan - 1) / kSpan, spans_all = spans_first + (pos - lo) / kSpan + 1;
   // with scratch for partial results a block takes one span (grid.z of them), else all of them in turn
   const int span_lo = part ? static_cast<int>(blockIdx.z) : 0, span_hi = part ? min(span_lo + 1, spans_all) : spans_all;
   if (span_lo >= span_hi) return;
-  for (int d = tid; d < dk; d += kThreads) qs[d] = to_float(q[(static_cast<size_t>(n) * nq + h) * dk + d]);
+  for (int i = tid; i < nh * dk; i += kThreads) qs[i / dk][i % dk] = to_float(q[(static_cast<size_t>(n) * nq + h0 + i / dk) * dk + i % dk]);
+  if (tid < kGroup) m_s[tid] = -INFINITY, l_s[tid] = 0.f;
   __syncthreads();
 
   const int groups = kThreads / dv;  // >= 1: dv <= 256
   const int g = tid / dv, d = tid % dv;
   const bool active = g < groups;
-  float m = -INFINITY, l = 0.f, acc = 0.f;
+  float acc[kGroup];
+#pragma unroll
+  for (int a = 0; a < kGroup; ++a) acc[a] = 0.f;
+  const int j = tid & (kSpan - 1), side = tid / kSpan;  // this thread's key of a span; it scores heads side, side + 2, ...
   for (int span = span_lo; span < span_hi; ++span) {
     const int base = span < spans_first ? span * kSpan : lo + (span - spans_first) * kSpan;
     const int cnt = min(kSpan, (span < spans_first ? kept_end : pos + 1) - base);
-    float lmax = -INFINITY;
-    for (int j = tid; j < cnt; j += kThreads) {
+    if (side < nh) {
       const int key = base + j;
-      const int page = table[key / page_size], off = key % page_size;
-      float s = -INFINITY;
-      row_s[j] = page >= 0 ? page * page_size + off : -1;  // the key's row in the cache, for the second product
+      const int page = j < cnt ? table[key / page_size] : -1, off = key % page_size;
+      float s[kGroup / 2];
+#pragma unroll
+      for (int a = 0; a < kGroup / 2; ++a) s[a] = 0.f;
+      if (side == 0) row_s[j] = page >= 0 ? page * page_size + off : -1;  // the key's row in the cache, for the second product
       if (page >= 0) {
         const T* kp = k_cache + ((static_cast<size_t>(page) * nkv + kvh) * page_size + off) * dk;
-        s = 0.f;
         if (VEC) {
-#pragma unroll 4
+#pragma unroll 2
           for (int e = 0; e < dk; e += 8) {
             float kv[8];
             load8(kp + e, kv);
 #pragma unroll
-            for (int u = 0; u < 8; ++u) s = fmaf(qs[e + u], kv[u], s);
+            for (int a = 0; a < kGroup / 2; ++a)
+              if (side + 2 * a < nh)
+#pragma unroll
+                for (int u = 0; u < 8; ++u) s[a] = fmaf(qs[side + 2 * a][e + u], kv[u], s[a]);
           }
         } else {
-          for (int e = 0; e < dk; ++e) s = fmaf(qs[e], to_float(kp[e]), s);
+          for (int e = 0; e < dk; ++e) {
+            const float kv = to_float(kp[e]);
+#pragma unroll
+            for (int a = 0; a < kGroup / 2; ++a)
+              if (side + 2 * a < nh) s[a] = fmaf(qs[side + 2 * a][e], kv, s[a]);
+          }
         }
-        s = shaped_score(s, scale, cap, bias_row, pos - key, far);
       }
-      sc[j] = s;
-      lmax = fmaxf(lmax, s);
+#pragma unroll
+      for (int a = 0; a < kGroup / 2; ++a)
+        if (side + 2 * a < nh) {
+          const float* bias_row = bias ? bias + static_cast<size_t>(h0 + side + 2 * a) * (far + 1) : nullptr;
+          sc[side + 2 * a][j] = page >= 0 ? shaped_score(s[a], scale, cap, bias_row, pos - key, far) : -INFINITY;
+        }
     }
-    const float m_new = fmaxf(m, block_max(lmax, scratch));
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = expf(m - m_use);
-    m = m_new;
-    float lsum = 0.f;
-    for (int j = tid; j < cnt; j += kThreads) {
-      const float p = expf(sc[j] - m_use);
-      sc[j] = p;
-      lsum += p;
+    __syncthreads();
+    // a wave a head: the running maximum and sum, the scores turned into weights
+    for (int a = wave; a < nh; a += kThreads / kWave) {
+      const float s0 = sc[a][lane], s1 = sc[a][lane + kWave];
+      const float m_old = m_s[a], m_new = fmaxf(m_old, wave_max(fmaxf(s0, s1)));
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float p0 = expf(s0 - m_use), p1 = expf(s1 - m_use), alpha = expf(m_old - m_use);
+      sc[a][lane] = p0, sc[a][lane + kWave] = p1;
+      const float sum = wave_sum(p0 + p1);
+      if (lane == 0) m_s[a] = m_new, l_s[a] = l_s[a] * alpha + sum, alpha_s[a] = alpha;
     }
-    l = l * alpha + block_sum(lsum, scratch);  // its barriers publish sc[] and row_s[]
-    acc *= alpha;
+    __syncthreads();
     if (active) {
+#pragma unroll
+      for (int a = 0; a < kGroup; ++a)
+        if (a < nh) acc[a] *= alpha_s[a];
       // eight keys at a time, so that their values are on their way together
       for (int j0 = g; j0 < cnt; j0 += 8 * groups) {
         float vv[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-          const int j = j0 + u * groups;
-          const int row = j < cnt ? row_s[j] : -1;
+          const int jj = j0 + u * groups;
+          const int row = jj < cnt ? row_s[jj] : -1;
           vv[u] = row >= 0 ? to_float(v_cache[((static_cast<size_t>(row / page_size) * nkv + kvh) * page_size + row % page_size) * dv + d]) : 0.f;
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-          const int j = j0 + u * groups;
-          if (j < cnt) acc = fmaf(sc[j], vv[u], acc);
+          const int jj = j0 + u * groups;
+          if (jj < cnt)
+#pragma unroll
+            for (int a = 0; a < kGroup; ++a)
+              if (a < nh) acc[a] = fmaf(sc[a][jj], vv[u], acc[a]);
         }
       }
     }
-    __syncthreads();  // sc[] is read; the next span may write it
+    __syncthreads();  // sc[] and row_s[] are read; the next span may write them
   }
-  accs[tid] = active ? acc : 0.f;
+#pragma unroll
+  for (int a = 0; a < kGroup; ++a) accs[a][tid] = active && a < nh ? acc[a] : 0.f;
   __syncthreads();
-  if (tid < dv) {
+  for (int i = tid; i < nh * dv; i += kThreads) {
+    const int a = i / dv, dd = i % dv, h = h0 + a;
     float total = 0.f;
-    for (int gg = 0; gg < groups; ++gg) total += accs[gg * dv + tid];
+    for (int gg = 0; gg < groups; ++gg) total += accs[a][gg * dv + dd];
     if (part) {  // [token of the list][head][span][dv + 2]: unnormalised output, max, sum
       float* dst = part + ((static_cast<size_t>(blockIdx.x) * nq + h) * gridDim.z + blockIdx.z) * (dv + 2);
-      dst[tid] = total;
-      if (tid == 0) dst[dv] = m, dst[dv + 1] = l;
-      return;
+      dst[dd] = total;
+      if (dd == 0) dst[dv] = m_s[a], dst[dv + 1] = l_s[a];
+      continue;
     }
+    const float l = l_s[a];
     float f = (l > 0.f ? 1.f / l : 0.f) * out_scale;
     if (gate) f *= gate[static_cast<size_t>(n) * nq + h];
-    out[static_cast<size_t>(n) * out_ld + h * dv + tid] = from_float<T>(total * f);
+    out[static_cast<size_t>(n) * out_ld + h * dv + dd] = from_float<T>(total * f);
   }
 }
 
@@ -604,6 +852,37 @@ extern "C" int pyre_attn_biased_tile(const void* q, void* out, int out_ld, int d
   }
   const bool vec = dk % 8 == 0 && dv % 8 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(v_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0;
+  if (dt == kBF16 && vec) {  // the 16-bit instruction, scores and weights in 32 bits all the same
+    const int ldk = dkp + kPad16, ldv = kKeys + kPad16;
+    size_t lds16 = sizeof(bf16) * (static_cast<size_t>(kKeys + 4 * 32) * ldk + 32 * nvp * ldv);
+    lds16 = (lds16 + 15) / 16 * 16;
+    const int tab16 = lds16 + sizeof(int) * table_stride <= 48 * 1024 ? table_stride : 0;
+    lds16 += sizeof(int) * tab16;
+    const int bias16 = bias && lds16 + sizeof(float) * 4 * (far + 1) <= 52 * 1024 ? 1 : 0;
+    lds16 += bias16 ? sizeof(float) * 4 * (far + 1) : 0;
+#define PYRE_TILE16(NV)                                                                                                  \
+  do {                                                                                                                   \
+    static size_t raised = 64 * 1024;                                                                                    \
+    if (lds16 > raised) {                                                                                                \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_biased_tile16_kernel<NV>),                             \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds16)) != hipSuccess)        \
+        return fail("attn_biased_tile: the device refuses %zu bytes of LDS", lds16);                                     \
+      raised = lds16;                                                                                                    \
+    }                                                                                                                    \
+    hipLaunchKernelGGL((attn_biased_tile16_kernel<NV>), grid, dim3(kThreads), lds16, stream, static_cast<const bf16*>(q), \
+                       static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), static_cast<bf16*>(out),    \
+                       out_ld, gate, out_scale, tiles, positions, seq_of_token, block_table, table_stride, nq, nkv, dk,  \
+                       dkp, dv, page_size, scale, cap, bias, far, window, keep_first, chunk, tab16, bias16);             \
+  } while (0)
+    switch (nvp) {
+      case 1: PYRE_TILE16(1); break;
+      case 2: PYRE_TILE16(2); break;
+      case 4: PYRE_TILE16(4); break;
+      default: PYRE_TILE16(8); break;
+    }
+#undef PYRE_TILE16
+    return check_launch("attn_biased_tile");
+  }
   if (dt == kF32) {
     if (vec) { PYRE_TILE_NV(float, true) } else { PYRE_TILE_NV(float, false) }
   } else {
@@ -632,13 +911,15 @@ extern "C" int pyre_attn_biased_single(const void* q, void* out, int out_ld, int
   PYRE_REQUIRE(known_dtype(dt) && table_stride > 0 && window >= 0 && keep_first >= 0 && far >= 0 && chunk >= 0, "attn_biased_single: bad arguments");
   PYRE_REQUIRE(!part || (max_spans >= 1 && max_spans <= 65535), "attn_biased_single: %d spans are not a launch", max_spans);
   if (n <= 0) return 0;
-  const dim3 grid(n, nq, part ? max_spans : 1);
+  // the query heads of a key/value head in as few blocks of up to kGroup heads as hold them, equally many in each
+  const int rep = nq / nkv, hgroups = (rep + kGroup - 1) / kGroup, hg = (rep + hgroups - 1) / hgroups;
+  const dim3 grid(n, nkv * hgroups, part ? max_spans : 1);
 #define PYRE_SINGLE(VEC)                                                                                                 \
   PYRE_DISPATCH(dt, T,                                                                                                    \
       hipLaunchKernelGGL((attn_biased_single_kernel<T, VEC>), grid, dim3(kThreads), 0, stream,                            \
                          static_cast<const T*>(q), static_cast<const T*>(k_cache), static_cast<const T*>(v_cache),        \
                          static_cast<T*>(out), out_ld, gate, out_scale, tokens, positions, seq_of_token, block_table,     \
-                         table_stride, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first, chunk, part))
+                         table_stride, nq, nkv, dk, dv, page_size, scale, cap, bias, far, window, keep_first, chunk, hg, part))
   if (dk % 8 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0) {
     PYRE_SINGLE(true);
   } else {
