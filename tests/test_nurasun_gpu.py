@@ -456,6 +456,53 @@ def test_what_stands_between_the_input_product_and_attention(dtype):
             assert float((cc[slot // page, 0, slot % page].cpu().double() - rows[t]).abs().max()) < tol * float(rows.abs().max())
 
 
+@pytest.mark.parametrize("nq,nkv,dk,dv,chunk", [(4, 2, 64, 64, 0), (6, 1, 128, 128, 0), (3, 3, 24, 40, 37), (5, 1, 136, 136, 0)])
+def test_attention_over_pages_in_16_bits_is_the_32_bit_one_rounded_once(nq, nkv, dk, dv, chunk):
+    """Prompt tiles and single tokens of bfloat16 queries, keys and values against float64 on the same values: the
+    16-bit kernels multiply exactly and keep scores and weights in float32, so what is left is the rounding of the
+    output (two to the minus eight of a value's size), not that of the weights (which would grow with the scores)."""
+    from pyre_amd.hip import ops
+
+    g = torch.Generator().manual_seed(nq * dk)
+    page, n = 16, 150
+    pages = (n + page - 1) // page
+    q = (torch.randn(n, nq * dk, generator=g)).bfloat16()
+    k = (torch.randn(n, nkv, dk, generator=g)).bfloat16()
+    v = k if dk == dv else (torch.randn(n, nkv, dv, generator=g)).bfloat16()
+    order = torch.randperm(pages + 3, generator=g)[:pages].to(torch.int32)      # the request's pages lie anywhere
+    kc = torch.zeros(pages + 3, nkv, page, dk, dtype=torch.bfloat16)
+    vc = torch.zeros(pages + 3, nkv, page, dv, dtype=torch.bfloat16)
+    for t in range(n):
+        kc[order[t // page], :, t % page], vc[order[t // page], :, t % page] = k[t], v[t]
+    scale = 2.0 / dk ** 0.5
+    want = torch.zeros(n, nq, dv, dtype=P.F)
+    visible = P.same_chunk(chunk) if chunk else P.causal
+    for head in range(nq):
+        kv = head // (nq // nkv)
+        a = P.softmax_rows((q.double().view(n, nq, dk)[:, head] @ k.double()[:, kv].T) * scale, visible)
+        want[:, head] = a @ v.double()[:, kv]
+    want = want.reshape(n, -1)
+    dev = lambda t: t.to(DEV)  # noqa: E731
+    positions, seqs = torch.arange(n, dtype=torch.int32), torch.zeros(n, dtype=torch.int32)
+    tiles = torch.tensor([[t0, min(32, n - t0)] for t0 in range(0, n, 32)], dtype=torch.int32)
+    shape = (nq, nkv, dk, dv, page, scale, 0.0, None, 0, 0, 0)
+    kcd, vcd = dev(kc), dev(vc)
+    if dk == dv:
+        vcd = kcd                                                                # one tensor as keys and values
+    ulp = 2.0 ** -8
+    if dk <= ops.ATTN_BIASED_TILE_MAX_KEY_HEAD:
+        out = torch.zeros(n, nq * dv, device=DEV, dtype=torch.bfloat16)
+        ops.attn_biased_tile(dev(q), out, kcd, vcd, None, 1.0, dev(tiles), len(tiles), dev(positions), dev(seqs),
+                             dev(order.view(1, -1)), *shape, chunk=chunk)
+        assert bool(((out.cpu().double() - want).abs() <= ulp * want.abs() + 1e-6).all())
+    out = torch.zeros(n, nq * dv, device=DEV, dtype=torch.bfloat16)
+    spans = ops.attn_biased_spans(pages, page, 0, 0, chunk)
+    scratch = torch.empty(n * nq * spans * (dv + 2), device=DEV)
+    ops.attn_biased_single(dev(q), out, kcd, vcd, None, 1.0, None, n, dev(positions), dev(seqs), dev(order.view(1, -1)), *shape,
+                           scratch=scratch if spans > 1 else None, chunk=chunk)
+    assert bool(((out.cpu().double() - want).abs() <= ulp * want.abs() + 1e-6).all())
+
+
 # ----------------------------------------------------------------------------- the entry points
 
 
