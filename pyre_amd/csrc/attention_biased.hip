@@ -911,8 +911,20 @@ extern "C" int pyre_attn_biased_single(const void* q, void* out, int out_ld, int
   PYRE_REQUIRE(known_dtype(dt) && table_stride > 0 && window >= 0 && keep_first >= 0 && far >= 0 && chunk >= 0, "attn_biased_single: bad arguments");
   PYRE_REQUIRE(!part || (max_spans >= 1 && max_spans <= 65535), "attn_biased_single: %d spans are not a launch", max_spans);
   if (n <= 0) return 0;
-  // the query heads of a key/value head in as few blocks of up to kGroup heads as hold them, equally many in each
-  const int rep = nq / nkv, hgroups = (rep + kGroup - 1) / kGroup, hg = (rep + hgroups - 1) / hgroups;
+  // the query heads of a key/value head in blocks of up to kGroup heads, which read the keys and values once for all of
+  // them: as many heads a block as still leave two blocks for every compute unit (a head's sums do not depend on its
+  // block-mates), equally many in each
+  const int rep = nq / nkv, want = 2 * compute_units();
+  int hgroups = rep;
+  for (int g = (rep + kGroup - 1) / kGroup; g < rep; ++g)
+    if (static_cast<long>(n) * nkv * g * (part ? max_spans : 1) >= want) {
+      hgroups = g;
+      break;
+    }
+  const int hg = (rep + hgroups - 1) / hgroups;
+  hgroups = (rep + hg - 1) / hg;  // as the kernel counts them: blocks of hg heads may be fewer than were asked for
+  PYRE_REQUIRE(hg >= 1 && hg <= kGroup && hgroups * hg >= rep && (hgroups - 1) * hg < rep && static_cast<long>(nkv) * hgroups <= 65535,
+               "attn_biased_single: %d heads a key/value head do not go into %d blocks of %d", rep, hgroups, hg);
   const dim3 grid(n, nkv * hgroups, part ? max_spans : 1);
 #define PYRE_SINGLE(VEC)                                                                                                 \
   PYRE_DISPATCH(dt, T,                                                                                                    \

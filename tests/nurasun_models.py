@@ -67,3 +67,10 @@ WIDE = model(64, 64, [
     layer(latent(4, 32, 16, 136, 0.4), dense(96)),
     layer(attention(6, 1, 16, 0.7, chunk=33, rot=8, base=90.0), dense(40)),
 ], eps=1e-6, mult=1.0, softcap=0.0)
+
+#: sizes that are multiples of nothing, so that no kernel's form for whole 16-byte pieces takes them
+ODD = model(77, 50, [
+    layer(attention(3, 1, 10, 0.9, chunk=11, rot=6, base=40.0), moe(3, 2, 5, shared=3)),
+    layer(latent(3, 5, 7, 9, 1.4), dense(9)),
+    layer(latent(2, 3, 3, 9, 0.8, kv_from=1), moe(6, 1, 7)),
+], eps=1e-4, mult=0.6, softcap=4.0)

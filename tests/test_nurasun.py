@@ -16,7 +16,7 @@ from pyre_amd.registry import config_from_dict, get_architecture
 
 
 def test_config_is_chosen_by_its_name_and_round_trips():
-    for raw in (M.SMALL, M.ONES, M.WIDE):
+    for raw in (M.SMALL, M.ONES, M.WIDE, M.ODD):
         cfg = config_from_dict(raw)
         assert isinstance(cfg, NurasunConfig) and cfg.to_dict() == raw and config_from_dict(cfg.to_dict()) == cfg
     cfg = config_from_dict(M.SMALL)

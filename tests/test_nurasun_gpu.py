@@ -21,7 +21,7 @@ pytestmark = pytest.mark.gpu
 #: bounds on max |difference| / max |logit| of a position, fixed before the first run: float32 against the float64
 #: plain run; bfloat16 loosely, because the sharp softmax of these models amplifies the rounding of queries and keys
 TOL = {"float32": 2e-5, "bfloat16": 8e-2}
-MODELS = {"small": (M.SMALL, 11), "ones": (M.ONES, 12), "wide": (M.WIDE, 13)}
+MODELS = {"small": (M.SMALL, 11), "ones": (M.ONES, 12), "wide": (M.WIDE, 13), "odd": (M.ODD, 14)}
 DEV = "cuda:0"
 
 _made = {}
@@ -130,7 +130,8 @@ def test_every_layer_of_a_whole_prompt(name, folders):
 
 # (the model of single heads of one to six elements runs in float32 only: in 16 bits its logits are mostly rounding)
 @pytest.mark.parametrize("name,dtype,page", [("small", "float32", 8), ("small", "bfloat16", 16), ("small", "float32", 4),
-                                             ("ones", "float32", 4), ("wide", "float32", 16), ("wide", "bfloat16", 8)])
+                                             ("ones", "float32", 4), ("wide", "float32", 16), ("wide", "bfloat16", 8),
+                                             ("odd", "float32", 8), ("odd", "bfloat16", 4)])
 def test_prefill_decode_and_portions_agree_with_plain(name, dtype, page, folders):
     folder, cfg, w = folders[name]
     reqs = {r: random_ids(cfg["vocab"], n, seed=n) for r, n in (("a", 90), ("b", 1), ("c", 37))}
@@ -456,7 +457,8 @@ def test_what_stands_between_the_input_product_and_attention(dtype):
             assert float((cc[slot // page, 0, slot % page].cpu().double() - rows[t]).abs().max()) < tol * float(rows.abs().max())
 
 
-@pytest.mark.parametrize("nq,nkv,dk,dv,chunk", [(4, 2, 64, 64, 0), (6, 1, 128, 128, 0), (3, 3, 24, 40, 37), (5, 1, 136, 136, 0)])
+@pytest.mark.parametrize("nq,nkv,dk,dv,chunk", [(4, 2, 64, 64, 0), (6, 1, 128, 128, 0), (3, 3, 24, 40, 37), (5, 1, 136, 136, 0),
+                                                 (7, 1, 64, 64, 0), (14, 2, 32, 32, 50), (28, 1, 16, 16, 0)])
 def test_attention_over_pages_in_16_bits_is_the_32_bit_one_rounded_once(nq, nkv, dk, dv, chunk):
     """Prompt tiles and single tokens of bfloat16 queries, keys and values against float64 on the same values: the
     16-bit kernels multiply exactly and keep scores and weights in float32, so what is left is the rounding of the
@@ -501,6 +503,13 @@ def test_attention_over_pages_in_16_bits_is_the_32_bit_one_rounded_once(nq, nkv,
     ops.attn_biased_single(dev(q), out, kcd, vcd, None, 1.0, None, n, dev(positions), dev(seqs), dev(order.view(1, -1)), *shape,
                            scratch=scratch if spans > 1 else None, chunk=chunk)
     assert bool(((out.cpu().double() - want).abs() <= ulp * want.abs() + 1e-6).all())
+    # some of the tokens only: other numbers of blocks, so other numbers of heads to a block, and the same rows
+    for count in (60, 33, 7):
+        some = torch.arange(n - count, n, dtype=torch.int32)
+        out2 = torch.zeros(n, nq * dv, device=DEV, dtype=torch.bfloat16)
+        ops.attn_biased_single(dev(q), out2, kcd, vcd, None, 1.0, dev(some), count, dev(positions), dev(seqs),
+                               dev(order.view(1, -1)), *shape, scratch=scratch if spans > 1 else None, chunk=chunk)
+        assert torch.equal(out2[n - count:], out[n - count:]) and not bool(out2[:n - count].any())
 
 
 # ----------------------------------------------------------------------------- the entry points
