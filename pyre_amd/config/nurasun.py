@@ -17,6 +17,14 @@ from pyre_amd.config.mafurax import _get, _positive_int
 from pyre_amd.config.model import ConfigError, ModelConfig
 
 
+def _scale(raw, dim: int, where: str) -> float:
+    """The factor on the scores: the configuration's, or 1 / sqrt(dim) where it names none."""
+    scale = float(_get(raw, "scale", where)) if "scale" in raw else dim ** -0.5
+    if not (scale > 0):
+        raise ConfigError(f"config.json: {where}.scale must be positive")
+    return scale
+
+
 @dataclass(frozen=True)
 class TiedAttentionConfig:
     """'attention': grouped heads, values tied to the keys, rotation of part of a head, runs of positions."""
@@ -32,7 +40,8 @@ class TiedAttentionConfig:
 
     @classmethod
     def from_dict(cls, raw, where):
-        heads, kv = _positive_int(raw, "heads", where), _positive_int(raw, "kv_heads", where)
+        heads = _positive_int(raw, "heads", where)
+        kv = _positive_int(raw, "kv_heads", where) if "kv_heads" in raw else heads   # not mentioned: a key head per query head
         if heads % kv:
             raise ConfigError(f"config.json: {where}.heads ({heads}) is not a multiple of kv_heads ({kv})")
         dim = _positive_int(raw, "dim", where)
@@ -46,7 +55,7 @@ class TiedAttentionConfig:
         base = float(rot.get("base", 10000.0))
         if dims and not (base > 0):
             raise ConfigError(f"config.json: {where}.rot.base must be positive")
-        return cls(heads, kv, dim, vdim, float(_get(raw, "scale", where)), chunk, dims, base)
+        return cls(heads, kv, dim, vdim, _scale(raw, dim, where), chunk, dims, base)
 
     def to_dict(self):
         out: dict[str, Any] = {"dim": self.dim, "heads": self.heads, "kv_heads": self.kv_heads, "scale": self.scale,
@@ -74,8 +83,9 @@ class LatentAttentionConfig:
         src = raw.get("kv_from")
         if src is not None and (isinstance(src, bool) or not isinstance(src, int) or src < 0):
             raise ConfigError(f"config.json: {where}.kv_from must name a layer, got {src!r}")
-        return cls(_positive_int(raw, "heads", where), _positive_int(raw, "dim", where), _positive_int(raw, "vdim", where),
-                   _positive_int(raw, "kv_rank", where), float(_get(raw, "scale", where)), src)
+        dim = _positive_int(raw, "dim", where)
+        return cls(_positive_int(raw, "heads", where), dim, _positive_int(raw, "vdim", where) if "vdim" in raw else dim,
+                   _positive_int(raw, "kv_rank", where), _scale(raw, dim, where), src)
 
     def to_dict(self):
         out: dict[str, Any] = {"dim": self.dim, "heads": self.heads, "kv_rank": self.kv_rank, "scale": self.scale,
