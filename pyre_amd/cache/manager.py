@@ -280,13 +280,15 @@ class CacheManager:
         if req.length > req.reserved:
             raise RuntimeError(f"request {rid!r}: committed past the reservation")
         for g, table, arr in zip(self.page_groups, req.tables, req.arrays):
-            w = g.spec.window
-            if w <= 0:
+            w, run = g.spec.window, getattr(g.spec, "chunk", 0)
+            if w <= 0 and run <= 0:
                 continue
-            # The next query sits at position req.length and sees keys > length - w.
-            dead_upto = req.length - w  # keys <= dead_upto are never read again
+            # The next query sits at position req.length and sees keys > length - w, and none before its own run
+            # of positions.
+            first_seen = max(req.length - w + 1 if w > 0 else 0, req.length - req.length % run if run > 0 else 0)
+            dead_upto = first_seen - 1  # keys <= dead_upto are never read again
             last_dead_page = (dead_upto + 1) // self.page_size - 1
-            kept_pages = -(-g.spec.keep_first // self.page_size)  # they hold the first tokens, which stay visible
+            kept_pages = -(-g.spec.keep_first // self.page_size) if w > 0 else 0  # they hold the first tokens, which stay visible
             dead = []
             for i in range(kept_pages, min(last_dead_page + 1, len(table))):
                 if table[i] != RELEASED:

@@ -112,7 +112,9 @@ class PagedTensorSpec:
 class PagedCacheSpec:
     """What a mixer keeps per token: one or more tensors in pages that share a block
     table. ``window`` = 0 keeps every token; ``window`` = W keeps the last W (a query at
-    position p sees p-W+1 .. p), and pages that no later query can see are given back."""
+    position p sees p-W+1 .. p), and pages that no later query can see are given back. ``chunk`` = C > 0:
+    a query sees only the keys of its own run of C positions (runs counted from position 0), so the pages
+    that lie wholly before the run of the next query are given back as well."""
 
     tensors: tuple[PagedTensorSpec, ...]
     window: int = 0
@@ -123,6 +125,8 @@ class PagedCacheSpec:
     #: whatever the engine is set to. All page groups of an engine share one page size, so an
     #: engine set to another size refuses the model when it is built.
     page_size: int | None = None
+    #: runs of this many positions: a query sees no key before its own run (0: no runs)
+    chunk: int = 0
 
     kind: ClassVar[str] = "paged"
 
@@ -130,8 +134,8 @@ class PagedCacheSpec:
         names = [t.name for t in self.tensors]
         if not names or len(names) != len(set(names)):
             raise ValueError("a paged cache needs at least one tensor, each with a name of its own")
-        if self.window < 0 or self.keep_first < 0:
-            raise ValueError("window and keep_first must not be negative")
+        if self.window < 0 or self.keep_first < 0 or self.chunk < 0:
+            raise ValueError("window, keep_first and chunk must not be negative")
         if self.page_size is not None and self.page_size <= 0:
             raise ValueError("page_size must be positive")
 

@@ -62,7 +62,7 @@ class TiedAttention(Mixer):
     def cache_spec(self):
         s = self.spec
         return PagedCacheSpec((PagedTensorSpec("k", (s.num_kv_heads, s.head_dim), token_axis=1),
-                               PagedTensorSpec("v", (s.num_kv_heads, s.head_dim), token_axis=1)))
+                               PagedTensorSpec("v", (s.num_kv_heads, s.head_dim), token_axis=1)), chunk=s.chunk)
 
     def step_arrays(self):
         return list(STEP_ARRAYS)

@@ -188,6 +188,40 @@ def test_a_window_gives_pages_back_once_passed():
     assert all(g.allocator.num_used == 0 for g in m.page_groups)
 
 
+def test_runs_of_positions_give_pages_back_when_a_run_ends():
+    """A group whose queries see their own run of positions only: pages that lie wholly before the next query's run
+    go back, for every way of cutting a request into portions every visible key is still held when its portion
+    runs, and a group without runs beside it keeps everything."""
+    runs = PagedCacheSpec((PagedTensorSpec("k", (2, 16), 1), PagedTensorSpec("v", (2, 16), 1)), chunk=40)
+    m = CacheManager([FULL, runs], 16, 12, 2, 512)
+    m.add_request("a")
+    m.reserve("a", 100)
+    m.commit("a", 100)
+    full, held = m.block_table("a", 0), m.block_table("a", 1)
+    # the next query at 100 is in the run 80..119: keys <= 79 are dead: pages 0..4 (keys 0..79) go
+    assert held[:5] == [RELEASED] * 5 and all(p != RELEASED for p in held[5:]) and RELEASED not in full
+    m.free_request("a")
+    assert all(g.allocator.num_used == 0 for g in m.page_groups)
+    rng = random.Random(5)
+    for _ in range(50):
+        c, ps = rng.choice([1, 5, 16, 33, 100]), rng.choice([4, 16])
+        m = CacheManager([PagedCacheSpec((PagedTensorSpec("k", (1, 8), 1),), chunk=c)], ps, 64, 1, 400)
+        m.add_request(0)
+        total = 0
+        while total < 300:
+            n = rng.choice([1, 1, 2, 7, 40])
+            m.reserve(0, n)
+            table = m.block_table(0, 0)
+            for key in range(total - total % c, total + n):      # the first query's run starts there
+                assert table[key // ps] != RELEASED
+            m.commit(0, n)
+            total += n
+            assert m.page_groups[0].allocator.num_used <= -(-(c + ps) // ps) + 1
+        m.check_invariants()
+        m.free_request(0)
+        assert m.page_groups[0].allocator.num_used == 0
+
+
 def test_window_release_never_hides_a_visible_key():
     """For every way of cutting a request into portions, each query's window
     [p - w + 1, p] lies in pages that are still held when the portion runs."""

@@ -61,6 +61,7 @@ def test_manifest_names_shapes_and_caches():
     caches = model.cache_specs()
     assert [len(c) for c in caches] == [1, 1, 0, 1, 1] and all(isinstance(c[0], PagedCacheSpec) for c in caches if c)
     assert [t.name for t in caches[0][0].tensors] == ["k", "v"] and caches[0][0].tensors[0].token_shape == (2, 24)
+    assert caches[0][0].chunk == 20 and caches[3][0].chunk == 7 and caches[1][0].chunk == 0
     assert [t.token_shape for t in caches[1][0].tensors] == [(1, 40)] and caches[4][0].tensors[0].token_shape == (1, 12)
     assert [c.cache_from for c in model.schedule] == [None, None, 1, None, None]
 

@@ -191,6 +191,19 @@ def test_long_decoding_across_many_runs_of_positions(folders):
     assert all_given_back(eng)
 
 
+def test_long_decoding_in_a_pool_that_only_ended_runs_make_fit():
+    """260 tokens one by one through a model whose layers all see runs of positions: the pages of a run go back when
+    the next run begins, so a pool of 64 tokens is enough (freed pages are filled with NaN: a read of one would show)."""
+    raw = M.model(113, 40, [M.SMALL["layers"][0], M.SMALL["layers"][3]], eps=1e-5, mult=0.45, softcap=9.0)
+    folder, cfg, w = _folder_of(raw, 21)
+    ids = random_ids(cfg["vocab"], 260, seed=1)
+    want = {"a": plain_rows(cfg, w, ids)}
+    eng = engine_of(folder, "float32", page_size=8, max_cached_tokens=64, max_model_len=512, debug_poison=True)
+    assert_close(replay(eng, one_by_one({"a": ids}, 2)), want, TOL["float32"])
+    assert_close(replay(eng, in_portions({"a": ids}, [5, 2, 19, 1, 7, 30])), want, TOL["float32"])
+    assert all_given_back(eng)
+
+
 # ----------------------------------------------------------------------------- keys made to stand out
 
 
