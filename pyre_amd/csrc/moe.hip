@@ -2,7 +2,8 @@
 //
 //   route_topk   z = the router product's partial sums, s = sigmoid(z); per token the `top` experts of largest
 //                s (the lower index among equals), each weighted s / (sum of the chosen s + 1e-20); written as a
-//                dense row gates[n, experts] (0 for an expert that is not chosen), float32.
+//                dense row gates[n, experts] (0 for an expert that is not chosen), float32. The experts are compared
+//                by z, which orders them as s does and still tells two apart where both their s round to one.
 //   expert_act   the experts' way up is one product over [W_0; W_1; ...; W_shared]; its result becomes
 //                act[n, e ff + j] = gates[n, e] f(up[n, e ff + j]) for the routed experts and f(up) for the columns
 //                of the shared expert behind them, f(u) = max(u, 0)^2. One product over
@@ -24,21 +25,21 @@ __global__ __launch_bounds__(kWave) void route_topk_kernel(const void* __restric
                                                            size_t partial_stride, const void* __restrict__ bias,
                                                            int bias_dt, float* __restrict__ gates, int experts, int top) {
   const int n = blockIdx.x, lane = threadIdx.x;
-  float s[kMaxPerLane], w[kMaxPerLane];
+  float s[kMaxPerLane], w[kMaxPerLane];  // s: the logits still to choose from
 #pragma unroll
   for (int u = 0; u < kMaxPerLane; ++u) {
     const int e = lane + kWave * u;
-    s[u] = -1.f, w[u] = 0.f;  // a sigmoid is never negative
+    s[u] = -INFINITY, w[u] = 0.f;
     if (e < experts) {
       float v = 0.f;
       for (int p = 0; p < n_partials; ++p) v += load_as_float(z, z_dt, p * partial_stride + static_cast<size_t>(n) * experts + e);
       if (bias) v += load_as_float(bias, bias_dt, e);
-      s[u] = 1.f / (1.f + expf(-v));
+      s[u] = fmaxf(v, -3.0e38f);  // finite, so that it beats the mark of an expert that is taken or not there
     }
   }
   float total = 0.f;
   for (int k = 0; k < top; ++k) {
-    float best = -1.f;
+    float best = -INFINITY;
     int at = experts;
 #pragma unroll
     for (int u = 0; u < kMaxPerLane; ++u)
@@ -49,10 +50,11 @@ __global__ __launch_bounds__(kWave) void route_topk_kernel(const void* __restric
       const int oa = __shfl_xor(at, o, kWave);
       if (ob > best || (ob == best && oa < at)) best = ob, at = oa;
     }
-    total += best;
+    const float score = 1.f / (1.f + expf(-best));
+    total += score;
 #pragma unroll
     for (int u = 0; u < kMaxPerLane; ++u)
-      if (at == lane + kWave * u) w[u] = best, s[u] = -1.f;
+      if (at == lane + kWave * u) w[u] = score, s[u] = -INFINITY;
   }
   const float inv = 1.f / (total + 1e-20f);
 #pragma unroll

@@ -412,6 +412,21 @@ def test_routing_and_the_experts_activation(experts, top, parts):
     assert float((act.cpu().double() - total).abs().max()) < 1e-5 * float(total.abs().max())
 
 
+def test_routing_tells_experts_apart_whose_scores_round_to_one():
+    """Logits of 15 to 40: their sigmoids are all 1 in float32, the experts are still chosen by the larger logit."""
+    from pyre_amd.hip import ops
+
+    g = torch.Generator().manual_seed(3)
+    n, experts, top = 9, 12, 3
+    z = 15 + 25 * torch.rand(n, experts, generator=g)
+    gates = torch.zeros(n, experts, device=DEV)
+    ops.route_topk(ops.Partials(z[None].contiguous().to(DEV)), gates, n, top)
+    chosen = (gates.cpu() > 0)
+    want = torch.zeros(n, experts, dtype=torch.bool)
+    want.scatter_(1, z.double().topk(top, dim=1).indices, True)
+    assert torch.equal(chosen, want) and float((gates.cpu().sum(1) - 1).abs().max()) < 1e-6
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("n,heads,din,dout", [(1, 3, 7, 19), (37, 5, 40, 24), (70, 2, 136, 300)])
 def test_the_product_per_head(dtype, n, heads, din, dout):
